@@ -7,7 +7,9 @@ paged caches fall into *groups* by what they need (their spec: widths, window). 
 every request has one block table per group; all caches of a group share the table (page p means page p of every
 cache's tensors).  Block table entry i covers positions [i * page_size, (i + 1) * page_size) of the request.
 A group with a window gives a page back as soon as every position in it lies behind the window of the
-next token to be computed; its table keeps a -1 there.  Pages return to the pool when a request is
+next token to be computed; its table keeps a -1 there.  A group whose rows stand for `every` > 1 positions each (`PagedSpec.every`:
+what a mixer keeps per block of tokens) has ceil(length / every) rows per request; entry i of its table covers the rows
+[i * page_size, (i + 1) * page_size).  Pages return to the pool when a request is
 released and are used again by later requests.  The reference has one pool, one table per sequence,
 no window and no state (ginfer/engine/block_manager.cc:63-148, ginfer/engine/model_runner.cc:52-87).
 
@@ -49,6 +51,15 @@ class _Request:
 def _block_tokens(token_ids, block, page_size):
     """The tokens of one full block as a key: their 32-bit values as bytes (compact, and compared exactly)."""
     return array("i", token_ids[block * page_size:(block + 1) * page_size]).tobytes()
+
+
+def _element_size(spec, default):
+    """Bytes of an element of a group's pages: the spec's own number format, or the model's."""
+    dtype = getattr(spec, "dtype", None)
+    if dtype is None:
+        return default
+    import torch
+    return torch.empty(0, dtype=dtype).element_size()
 
 
 def _is_paged(spec):
@@ -105,6 +116,15 @@ class CacheGroup:
     def window(self):
         return self.spec.window
 
+    @property
+    def every(self):
+        """Positions that one row of this group's pages stands for (1: a row a token)."""
+        return int(getattr(self.spec, "every", 1))
+
+    def rows_for(self, tokens):
+        """Rows that a request of this many tokens holds."""
+        return -(-tokens // self.every)
+
     def first_needed_block(self, next_pos):
         """Blocks before this one hold only positions that no query at or after next_pos can see."""
         if self.window is None:
@@ -152,6 +172,7 @@ class CacheManager:
         self._table_np = [np.full((self.max_requests, 16), -1, dtype=np.int32) for _ in self.groups]
         self._length_np = np.zeros(self.max_requests, dtype=np.int64)
         self._any_window = any(g.window is not None for g in self.groups)
+        self._any_stride = any(g.every > 1 for g in self.groups)
 
     @staticmethod
     def group_specs(cache_specs):
@@ -200,8 +221,9 @@ class CacheManager:
         groups = cls.group_specs(cache_specs)
         if not groups:
             return []
-        page_bytes = [len(units) * sum(w for _, w in spec.page_tensors()) * page_size * element_size
+        page_bytes = [len(units) * sum(w for _, w in spec.page_tensors()) * page_size * _element_size(spec, element_size)
                       for spec, units in groups.items()]
+        every = [int(getattr(spec, "every", 1)) for spec in groups]
         counts, left = [None] * len(groups), int(pool_bytes)
         for gi, spec in enumerate(groups):
             if spec.window is not None:
@@ -209,9 +231,12 @@ class CacheManager:
                 left -= counts[gi] * page_bytes[gi]
         rest = [gi for gi, c in enumerate(counts) if c is None]
         if rest:
-            per = left // sum(page_bytes[gi] for gi in rest) if left > 0 else 0
+            # a group whose rows stand for several positions needs that many fewer pages for the same tokens, and one more
+            # per request for the block that is not full yet
+            extra = sum(page_bytes[gi] * (max_requests + 1) for gi in rest if every[gi] > 1)
+            per = int((left - extra) // sum(page_bytes[gi] / every[gi] for gi in rest)) if left > extra else 0
             for gi in rest:
-                counts[gi] = per
+                counts[gi] = per if every[gi] == 1 else per // every[gi] + max_requests + 1
         elif left < 0:       # windows only and too little memory: shrink them alike
             total = sum(c * b for c, b in zip(counts, page_bytes))
             counts = [c * int(pool_bytes) // total for c in counts]
@@ -229,13 +254,14 @@ class CacheManager:
     # ---- device memory
     def pool_bytes(self, element_size):
         return sum(g.pool.num_pages * len(g.units) * sum(w for _, w in g.spec.page_tensors()) * self.page_size
-                   * element_size for g in self.groups)
+                   * _element_size(g.spec, element_size) for g in self.groups)
 
     def allocate_device(self, dtype, device):
         import torch
         for g in self.groups:
-            g.tensors = {name: torch.zeros((len(g.units), g.pool.num_pages, self.page_size * width), dtype=dtype,
-                                           device=device) for name, width in g.spec.page_tensors()}
+            g.tensors = {name: torch.zeros((len(g.units), g.pool.num_pages, self.page_size * width),
+                                           dtype=getattr(g.spec, "dtype", None) or dtype, device=device)
+                         for name, width in g.spec.page_tensors()}
         for unit in self.state_units:
             s = caches_of(self.cache_specs[unit[0]])[unit[1]]
             self.state_tensors[unit] = torch.zeros((self.max_requests + 1,) + tuple(s.shape), dtype=s.dtype, device=device)
@@ -340,9 +366,9 @@ class CacheManager:
         """Per group: (blocks to give back, pages to take) for n_new more tokens."""
         plan = []
         start, end = req.length, req.length + n_new
-        need_blocks = -(-end // self.page_size)
         for gi, g in enumerate(self.groups):
             table = req.tables[gi]
+            need_blocks = -(-g.rows_for(end) // self.page_size)
             if g.window is None:         # a table without a window has no gaps: what is missing lies at its end
                 plan.append(([], max(0, need_blocks - len(table)), 0, need_blocks))
                 continue
@@ -377,6 +403,10 @@ class CacheManager:
             first = g.first_needed_block(req.length)
             give = sum(1 for i in range(req.gone[gi], min(first, len(table))) if table[i] >= 0)
             have_blocks = len(table)
+            if g.every > 1:      # rows of `every` positions: what the pages at hand and the free ones hold, less what is used
+                cap = max(0, (have_blocks + g.pool.num_free) * self.page_size * g.every - req.length)
+                best = cap if best is None else min(best, cap)
+                continue
             room = have_blocks * self.page_size - req.length if have_blocks * self.page_size > req.length else 0
             cap = room + (g.pool.num_free + give) * self.page_size
             best = cap if best is None else min(best, cap)
@@ -401,7 +431,7 @@ class CacheManager:
         return first
 
     def _append(self, req, rid, n_new):
-        if n_new == 1 and not self._any_window and req.length % self.page_size:
+        if n_new == 1 and not self._any_window and not self._any_stride and req.length % self.page_size:
             req.pending = 1              # the common decode step: room is left in the last page
             return req.length
         plan = self._plan(req, n_new)

@@ -4,7 +4,8 @@ from .spec import PartSpec, LayerSpec, prenorm_layer, ScheduleEntry, ModelSpec
 from .qwen2 import Qwen2Config
 from .titozen import TitozenConfig
 from .potupel import PotupelConfig
+from .puguzen import PuguzenConfig
 
 __all__ = ["ConfigError", "register_architecture", "registered_architectures", "config_class",
            "config_from_dict", "config_from_folder", "PartSpec", "LayerSpec", "prenorm_layer", "ScheduleEntry",
-           "ModelSpec", "Qwen2Config", "TitozenConfig"]
+           "ModelSpec", "Qwen2Config", "TitozenConfig", "PotupelConfig", "PuguzenConfig"]

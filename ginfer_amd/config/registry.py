@@ -58,4 +58,7 @@ def config_from_folder(folder):
             d = json.load(f)
         except json.JSONDecodeError as e:
             raise ConfigError("%s is not valid JSON: %s" % (path, e))
-    return config_from_dict(d)
+    config = config_from_dict(d)
+    # a family whose config.json leaves a size to the tensors' shapes reads it from the folder's checkpoint
+    read = getattr(config, "read_folder", None)
+    return read(folder) if read is not None else config

@@ -129,6 +129,7 @@ template <typename T>
 __device__ __forceinline__ float clamped_glu_one(float g, float u, float limit, float alpha, float shift) {
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
+  if (isinf(alpha)) return (g > 0.f ? g : 0.f) * (u + shift);     // the sigmoid's limit, a step at zero: relu(g)
   return (g * (1.0f / (1.0f + expf(-alpha * g)))) * (u + shift);
 }
 

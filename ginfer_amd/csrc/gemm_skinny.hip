@@ -172,13 +172,15 @@ struct KRange {
 // silu(gate) * up = (g * (1 / (1 + exp(-g)))) * u (ginfer/core/op/kernels/cuda/swiglu_kernel.cu:24-27) for N
 // columns: the activation of the feed-forward without a pass over memory of its own.
 // The gate of a gated product: out = g * sigmoid(alpha g) * (u + shift) with g = min(gate, limit) and u = clamp(up, -limit,
-// limit).  limit = infinity, alpha = 1, shift = 0 is SiLU(gate) * up, bit for bit what stood here before the bounds.
+// limit).  limit = infinity, alpha = 1, shift = 0 is SiLU(gate) * up, bit for bit what stood here before the bounds; alpha =
+// infinity stands for the sigmoid's limit, a step at zero: relu(g) * (u + shift).
 struct GateAct {
   float limit, alpha, shift;
 };
 __device__ __forceinline__ float gate_act(float v, float u, const GateAct act) {
   v = fminf(v, act.limit);
   u = fminf(fmaxf(u, -act.limit), act.limit);
+  if (isinf(act.alpha)) return (v > 0.f ? v : 0.f) * (u + act.shift);     // the sigmoid's limit, a step: relu(g)
   return (v * (1.0f / (1.0f + expf(-(act.alpha * v))))) * (u + act.shift);
 }
 

@@ -228,6 +228,45 @@ int ga_combine_pairs(void* out, const void* y, const void* shared, const void* w
 // ---- activation.hip: out[i] = max(x[i], 0)^2 over `total` elements (out may be x)
 int ga_relu_square(void* out, const void* x, int64_t total, int is_bf16, hipStream_t stream);
 
+// ---- decay_scan.hip: linear attention with a decay as a recurrence, S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per
+// head.  q, k, v: 32-bit rows with a common stride; a from `decay` float [tokens, heads dim] or from `head_decay` float
+// [heads] (exactly one of them); q and k turned on their first rot_dims coordinates (pairs i, i + rot_dims / 2; tables float
+// [positions, rot_dims / 2]) and multiplied by q_scale, k_scale; state float [slots, heads, dim, vdim], zeros for a request
+// whose q_start is 0; out float [tokens, heads, vdim]
+int ga_decay_scan(void* out, const void* q, const void* k, const void* v, int64_t stride, const void* decay,
+                  const void* head_decay, const void* cos_t, const void* sin_t, int rot_dims, float q_scale, float k_scale,
+                  void* state, const void* slots, const void* cu, const void* q_start, int entries, int heads, int dim,
+                  int vdim, hipStream_t stream);
+// decay float [tokens, channels] = sigmoid(a2 low + bias)^(1 / tau); low: 32-bit rows of `rank` numbers with a stride; a2
+// float [channels, rank]
+int ga_gla_decay(void* decay, const void* low, int64_t low_stride, const void* a2, const void* bias, int tokens,
+                 int channels, int rank, float tau, hipStream_t stream);
+// out [tokens, heads, vdim] = x / rms(x over vdim) (* weight [vdim], or null) (* silu(gate), 32-bit rows with a stride, or null)
+int ga_head_norm_gate(void* out, const void* x, const void* weight, const void* gate, int64_t gate_stride, int64_t tokens,
+                      int heads, int vdim, float eps, int out_bf16, hipStream_t stream);
+
+// ---- pooled_attention.hip: attention over a window of tokens and the means of the blocks before it, sigmoid weights.
+// prepare: q and k of a 32-bit projection [q heads | k heads | v heads ...] turned by position (pairs 2i, 2i + 1), divided by
+// their root mean square per head where `unit`; q out float [tokens, nh dim]; k, v into rows [slot][nkv][dim | vdim]
+int ga_pwa_prepare(void* q_out, const void* proj, int64_t stride, const void* positions, const void* cos_t, const void* sin_t,
+                   const void* slot_mapping, void* k_rows, void* v_rows, int tokens, int nh, int nkv, int dim, int vdim,
+                   int rot_dims, int unit, float eps, int write, int cache_bf16, hipStream_t stream);
+// for every token that ends a block of `pool` positions: the block's mean key and value (float rows at pool_slots[token])
+int ga_pwa_pool(void* pk_rows, void* pv_rows, const void* k_rows, const void* v_rows, const void* positions,
+                const void* token_entry, const void* table, int width, const void* pool_slots, int tokens, int nkv, int dim,
+                int vdim, int pool, int page_size, int cache_bf16, hipStream_t stream);
+// out [tokens, nh vdim] = sum over the visible blocks and tokens of sigmoid(scale q . k + head_bias) v (* sigmoid(gate))
+int ga_pwa_attend(void* out, const void* q, const void* k_rows, const void* v_rows, const void* pk_rows, const void* pv_rows,
+                  const void* positions, const void* token_entry, const void* table, int width, const void* pool_table,
+                  int pool_width, const void* head_bias, const void* gate, int64_t gate_stride, int tokens, int nh, int nkv,
+                  int dim, int vdim, int size, int pool, int page_size, float scale, int cache_bf16, int out_bf16,
+                  hipStream_t stream);
+
+// ---- gated_residual.hip: residual float [tokens, hidden] += sigmoid(z[:, :hidden]) * y1 (+ sigmoid(z[:, hidden:]) * y2, y2
+// may be null); with next: next = rmsnorm(residual) * next_gain (float [hidden])
+int ga_gated_residual_add(void* residual, const void* z, const void* y1, const void* y2, int tokens, int hidden, int y_bf16,
+                          const void* next_gain, float next_eps, void* next, int next_bf16, hipStream_t stream);
+
 // ---- random_fill.hip: out[i] = mean + std * normal(key, i) for n elements, float or bfloat16: the counter-based
 // generator of random_normal.h, which gives the host library (host/random_fill_host.cpp) the same bits
 int ga_random_normal_fill(void* out, int64_t n, uint64_t key, float mean, float std, int is_bf16, hipStream_t stream);

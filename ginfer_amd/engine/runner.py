@@ -254,11 +254,13 @@ class ModelRunner:
         tables, slot_maps = [], []
         for gi in range(len(cache.groups)):
             bt = cache.tables_array(gi, slots, width)
-            pages = bt[ent, pos // ps].astype(np.int64)
+            every = cache.groups[gi].every
+            row = pos if every == 1 else pos // every        # a group may keep a row per block of positions
+            pages = bt[ent, row // ps].astype(np.int64)
             if (pages < 0).any():
                 raise AssertionError("a new token has no page in cache group %d" % gi)
             tables.append(bt)
-            slot_maps.append(pages * ps + pos % ps)
+            slot_maps.append(pages * ps + row % ps)
         return dict(E=E, T=T, ids=ids.astype(np.int32), pos=pos, ent=ent, cu=cu, q_start=q_start.astype(np.int32),
                     q_len=q_len, rows=np.asarray(rows, dtype=np.int32), width=width, tables=tables,
                     slot_maps=slot_maps, state_slots=slots, max_kv=max_kv,

@@ -1230,3 +1230,228 @@ def conv_rope_kv(proj, weight, state, slots, step, cos, sin, slot_mapping, k_pag
                                _i(_is_bf16(proj.dtype)), _stream()),
            "conv_rope_kv")
     return q
+
+
+DECAY_SCAN_MAX_DIM = 256
+
+
+def _step_entries(step, slots):
+    E = step.cu_tokens.shape[0] - 1
+    for name, a, n in (("cu_tokens", step.cu_tokens, E + 1), ("q_start", step.q_start, E)):
+        _need(a.dtype == torch.int32 and a.shape == (n,) and a.is_contiguous(), "%s must be contiguous int32 [%d]", name, n)
+    _need(slots.dtype == torch.int64 and slots.shape == (E,) and slots.is_contiguous(), "slots must be contiguous int64 [%d]", E)
+    return E
+
+
+def _rows_of(proj, start, width, name):
+    """A block of columns of a 32-bit projection as (view, row stride)."""
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and 0 <= start and start + width <= proj.shape[1],
+          "%s: columns %d .. %d of a float32 projection with unit inner stride, got %s %s", name, start, start + width, proj.dtype,
+          tuple(proj.shape))
+    return proj[:, start:start + width]
+
+
+def gla_decay(proj, low_start, a2, bias, tau):
+    """sigmoid(a2 low + bias)^(1 / tau) in 32-bit: low = proj[:, low_start : low_start + rank] (float32 rows), a2 float32
+    [channels, rank], bias float32 [channels].  Returns float32 [T, channels]."""
+    _dev(proj, a2, bias)
+    _need(a2.dim() == 2, "a2 must be [channels, rank]")
+    C, R = a2.shape
+    _f32(a2, (C, R), "a2")
+    _f32(bias, (C,), "bias")
+    low = _rows_of(proj, low_start, R, "low")
+    _need(tau > 0, "tau must be positive, got %r", tau)
+    T = proj.shape[0]
+    out = torch.empty((T, C), dtype=torch.float32, device=proj.device)
+    lib = build.load("decay_scan")
+    _check(lib.ga_gla_decay(_ptr(out), _ptr(low), _i64(proj.stride(0)), _ptr(a2), _ptr(bias), _i(T), _i(C), _i(R), _f(tau),
+                            _stream()), "gla_decay")
+    return out
+
+
+def decay_scan(proj, q_start, k_start, v_start, state, slots, step, heads, dim, vdim, decay=None, head_decay=None, cos=None,
+               sin=None, q_scale=1.0, k_scale=1.0):
+    """Linear attention with a decay as a recurrence over per-request state: S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T
+    q_t per head.  q, k, v are column blocks of the float32 projection `proj` (starting at q_start, k_start, v_start; heads *
+    dim, heads * dim, heads * vdim wide).  a: `decay` float32 [T, heads * dim], or `head_decay` float32 [heads].  cos, sin
+    float32 [positions, r / 2]: q and k are turned on their first r coordinates (pairs i, i + r / 2) by the tokens' positions,
+    then multiplied by q_scale and k_scale.  state float32 [slots, heads, dim, vdim] is advanced in place (zeros where an
+    entry's q_start is 0).  Returns float32 [T, heads, vdim]."""
+    _dev(proj, state, slots, decay, head_decay, cos, sin)
+    T = proj.shape[0]
+    q = _rows_of(proj, q_start, heads * dim, "q")
+    k = _rows_of(proj, k_start, heads * dim, "k")
+    v = _rows_of(proj, v_start, heads * vdim, "v")
+    _need(0 < dim <= DECAY_SCAN_MAX_DIM, "the recurrence kernel takes up to %d key channels per head, got %d", DECAY_SCAN_MAX_DIM, dim)
+    _need((decay is None) != (head_decay is None), "the decay comes per token and channel, or per head: exactly one of the two")
+    if decay is not None:
+        _f32(decay, (T, heads * dim), "decay")
+    else:
+        _f32(head_decay, (heads,), "head_decay")
+    rot = 0
+    if cos is not None:
+        _need(sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape
+              and cos.dim() == 2 and cos.is_contiguous() and sin.is_contiguous(), "cos and sin must be contiguous float32 [P, r/2]")
+        rot = 2 * cos.shape[1]
+        _need(0 < rot <= dim, "the rotation covers %d coordinates of a head of %d", rot, dim)
+        _need(step.max_kv_len <= cos.shape[0], "positions up to %d, tables for %d", step.max_kv_len, cos.shape[0])
+    _need(state.dtype == torch.float32 and state.dim() == 4 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dim, vdim),
+          "state must be contiguous float32 [slots, %d, %d, %d]", heads, dim, vdim)
+    E = _step_entries(step, slots)
+    out = torch.empty((T, heads, vdim), dtype=torch.float32, device=proj.device)
+    lib = build.load("decay_scan")
+    _check(lib.ga_decay_scan(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _i64(proj.stride(0)), _ptr(decay), _ptr(head_decay),
+                             _ptr(cos), _ptr(sin), _i(rot), _f(q_scale), _f(k_scale), _ptr(state), _ptr(slots),
+                             _ptr(step.cu_tokens), _ptr(step.q_start), _i(E), _i(heads), _i(dim), _i(vdim), _stream()), "decay_scan")
+    return out
+
+
+def head_norm_gate(x, weight, eps, dtype, proj=None, gate_start=0):
+    """x float32 [T, heads, V] -> [T, heads * V] in `dtype`: every head's row divided by its root mean square, times weight
+    [V] (None: no weight), times silu of the gate, the columns gate_start .. gate_start + heads * V of the float32
+    projection `proj` (None: no gate)."""
+    _dev(x, weight, proj)
+    _need(x.dtype == torch.float32 and x.dim() == 3 and x.is_contiguous(), "x must be contiguous float32 [T, heads, V]")
+    T, H, V = x.shape
+    if weight is not None:
+        _f32(weight, (V,), "weight")
+    gate = None
+    if proj is not None:
+        _need(proj.shape[0] == T, "the gate has %d rows, x has %d", proj.shape[0], T)
+        gate = _rows_of(proj, gate_start, H * V, "gate")
+    out = torch.empty((T, H * V), dtype=dtype, device=x.device)
+    lib = build.load("decay_scan")
+    _check(lib.ga_head_norm_gate(_ptr(out), _ptr(x), _ptr(weight), _ptr(gate), _i64(proj.stride(0) if proj is not None else 0),
+                                 _i64(T), _i(H), _i(V), _f(eps), _i(_is_bf16(dtype)), _stream()), "head_norm_gate")
+    return out
+
+
+POOLED_ATTENTION_MAX_DIM = 256
+
+
+def _token_rows(t, width, name, dtype=None):
+    """A paged tensor viewed as rows of `width` elements, a slot a row."""
+    _need(t is not None and t.is_contiguous() and t.numel() % width == 0 and (dtype is None or t.dtype == dtype),
+          "%s must be contiguous%s and hold whole rows of %d", name, "" if dtype is None else " " + str(dtype), width)
+    return t.numel() // width
+
+
+def pooled_attention_prepare(proj, positions, cos, sin, slot_mapping, k_rows, v_rows, num_heads, num_kv_heads, dim, vdim, eps,
+                             unit_norm=True, write=True):
+    """Behind a float32 projection whose first columns are [q heads | k heads | v heads]: q and k turned by position on their
+    first r coordinates (pairs 2i, 2i + 1; cos, sin float32 [positions, r / 2], None: no rotation), then divided by their
+    root mean square per head (unit_norm); k and v are written into their rows ([slot][kv head][dim | vdim], float32 or
+    bfloat16) at slot_mapping.  Returns q float32 [T, num_heads * dim]."""
+    _dev(proj, positions, cos, sin, slot_mapping, k_rows, v_rows)
+    T = proj.shape[0]
+    _rows_of(proj, 0, (num_heads + num_kv_heads) * dim + num_kv_heads * vdim, "q | k | v")
+    _need(0 < dim <= POOLED_ATTENTION_MAX_DIM and 0 < vdim <= POOLED_ATTENTION_MAX_DIM, "heads of %d / %d are not supported: up to %d",
+          dim, vdim, POOLED_ATTENTION_MAX_DIM)
+    _need(positions.dtype == torch.int32 and positions.shape == (T,) and positions.is_contiguous(), "positions must be contiguous int32 [T]")
+    rot = 0
+    if cos is not None:
+        _need(sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape
+              and cos.dim() == 2 and cos.is_contiguous() and sin.is_contiguous(), "cos and sin must be contiguous float32 [P, r/2]")
+        rot = 2 * cos.shape[1]
+        _need(0 < rot <= dim, "the rotation covers %d coordinates of a head of %d", rot, dim)
+    cache_bf16 = 0
+    if write:
+        _need(slot_mapping.dtype == torch.int64 and slot_mapping.shape == (T,) and slot_mapping.is_contiguous(),
+              "slot_mapping must be contiguous int64 [T]")
+        _need(k_rows.dtype == v_rows.dtype, "keys and values are cached in one number format")
+        cache_bf16 = _is_bf16(k_rows.dtype)
+        _need(_token_rows(k_rows, num_kv_heads * dim, "k_rows") == _token_rows(v_rows, num_kv_heads * vdim, "v_rows"),
+              "keys and values must hold the same number of rows")
+    q = torch.empty((T, num_heads * dim), dtype=torch.float32, device=proj.device)
+    lib = build.load("pooled_attention")
+    _check(lib.ga_pwa_prepare(_ptr(q), _ptr(proj), _i64(proj.stride(0)), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
+                              _ptr(k_rows), _ptr(v_rows), _i(T), _i(num_heads), _i(num_kv_heads), _i(dim), _i(vdim), _i(rot),
+                              _i(1 if unit_norm else 0), _f(eps), _i(1 if write else 0), _i(cache_bf16), _stream()), "pwa_prepare")
+    return q
+
+
+def _table(t, entries, name):
+    _need(t.dtype == torch.int32 and t.dim() == 2 and t.shape[0] == entries and t.shape[1] >= 1 and t.is_contiguous(),
+          "%s must be contiguous int32 [%d, width]", name, entries)
+    return t.shape[1]
+
+
+def pooled_attention_pool(pk_rows, pv_rows, k_rows, v_rows, step, table, pool_slots, num_kv_heads, dim, vdim, pool, page_size):
+    """For every token of the step that ends a block of `pool` positions: the means of the block's cached keys and values
+    (read through the entries' block `table`) into the float32 rows pk_rows, pv_rows at pool_slots[token] (-1: none)."""
+    _dev(pk_rows, pv_rows, k_rows, v_rows, table, pool_slots)
+    T = step.positions.shape[0]
+    E = step.cu_tokens.shape[0] - 1
+    width = _table(table, E, "table")
+    _need(pool_slots.dtype == torch.int64 and pool_slots.shape == (T,) and pool_slots.is_contiguous(), "pool_slots must be contiguous int64 [T]")
+    _need(step.token_entry.dtype == torch.int32 and step.token_entry.shape == (T,), "token_entry must be int32 [T]")
+    _need(k_rows.dtype == v_rows.dtype, "keys and values are cached in one number format")
+    _token_rows(k_rows, num_kv_heads * dim, "k_rows")
+    _token_rows(v_rows, num_kv_heads * vdim, "v_rows")
+    _token_rows(pk_rows, num_kv_heads * dim, "pk_rows", torch.float32)
+    _token_rows(pv_rows, num_kv_heads * vdim, "pv_rows", torch.float32)
+    _need(pool >= 1 and page_size >= 1, "pool and page_size must be positive")
+    lib = build.load("pooled_attention")
+    _check(lib.ga_pwa_pool(_ptr(pk_rows), _ptr(pv_rows), _ptr(k_rows), _ptr(v_rows), _ptr(step.positions), _ptr(step.token_entry),
+                           _ptr(table), _i(width), _ptr(pool_slots), _i(T), _i(num_kv_heads), _i(dim), _i(vdim), _i(pool),
+                           _i(page_size), _i(_is_bf16(k_rows.dtype)), _stream()), "pwa_pool")
+
+
+def pooled_attention(q, k_rows, v_rows, pk_rows, pv_rows, step, table, pool_table, head_bias, num_heads, num_kv_heads, dim, vdim,
+                     size, pool, page_size, scale, dtype, proj=None, gate_start=0):
+    """q float32 [T, num_heads * dim].  Token i sees the tokens j with 0 <= i - j < size and the means of the blocks of `pool`
+    tokens that end before them; the weight of a key is sigmoid(scale q . k + head_bias[head]) (head_bias float32 [heads] or
+    None), not normalised.  The result is multiplied by sigmoid of the gate, the columns gate_start .. of the float32 projection
+    `proj` (None: no gate).  Returns [T, num_heads * vdim] in `dtype`."""
+    _dev(q, k_rows, v_rows, pk_rows, pv_rows, table, pool_table, head_bias, proj)
+    T = q.shape[0]
+    _f32(q, (T, num_heads * dim), "q")
+    E = step.cu_tokens.shape[0] - 1
+    width, pool_width = _table(table, E, "table"), _table(pool_table, E, "pool_table")
+    _need(num_heads % num_kv_heads == 0, "num_heads %d is not a multiple of num_kv_heads %d", num_heads, num_kv_heads)
+    _need(0 < dim <= POOLED_ATTENTION_MAX_DIM and 0 < vdim <= POOLED_ATTENTION_MAX_DIM, "heads of %d / %d are not supported: up to %d",
+          dim, vdim, POOLED_ATTENTION_MAX_DIM)
+    _need(k_rows.dtype == v_rows.dtype, "keys and values are cached in one number format")
+    _token_rows(k_rows, num_kv_heads * dim, "k_rows")
+    _token_rows(v_rows, num_kv_heads * vdim, "v_rows")
+    _token_rows(pk_rows, num_kv_heads * dim, "pk_rows", torch.float32)
+    _token_rows(pv_rows, num_kv_heads * vdim, "pv_rows", torch.float32)
+    for name, a in (("positions", step.positions), ("token_entry", step.token_entry)):
+        _need(a.dtype == torch.int32 and a.shape == (T,) and a.is_contiguous(), "%s must be contiguous int32 [T]", name)
+    if head_bias is not None:
+        _f32(head_bias, (num_heads,), "head_bias")
+    gate = None
+    if proj is not None:
+        _need(proj.shape[0] == T, "the gate has %d rows, q has %d", proj.shape[0], T)
+        gate = _rows_of(proj, gate_start, num_heads * vdim, "gate")
+    _need(size >= 1 and pool >= 1 and page_size >= 1, "size, pool and page_size must be positive")
+    out = torch.empty((T, num_heads * vdim), dtype=dtype, device=q.device)
+    lib = build.load("pooled_attention")
+    _check(lib.ga_pwa_attend(_ptr(out), _ptr(q), _ptr(k_rows), _ptr(v_rows), _ptr(pk_rows), _ptr(pv_rows), _ptr(step.positions),
+                             _ptr(step.token_entry), _ptr(table), _i(width), _ptr(pool_table), _i(pool_width), _ptr(head_bias),
+                             _ptr(gate), _i64(proj.stride(0) if proj is not None else 0), _i(T), _i(num_heads), _i(num_kv_heads),
+                             _i(dim), _i(vdim), _i(size), _i(pool), _i(page_size), _f(scale), _i(_is_bf16(k_rows.dtype)),
+                             _i(_is_bf16(dtype)), _stream()), "pwa_attend")
+    return out
+
+
+def gated_residual_add(residual, z, y1, y2=None, next_gain=None, next_eps=0.0, dtype=None):
+    """residual float32 [T, H] += sigmoid(z[:, :H]) * y1 (+ sigmoid(z[:, H:]) * y2), the gated results added to each other
+    first; z float32 [T, H] or [T, 2H]; y1, y2 [T, H] in float32 or bfloat16.  With next_gain (float32 [H]) the rows of the norm
+    that is read next, rmsnorm(residual) * next_gain in `dtype`, come back; else None."""
+    _dev(residual, z, y1, y2, next_gain)
+    _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(), "residual must be contiguous float32 [T, H]")
+    T, H = residual.shape
+    gates = 1 if y2 is None else 2
+    _f32(z, (T, gates * H), "z")
+    for name, y in (("y1", y1), ("y2", y2)):
+        _need(y is None or (y.shape == (T, H) and y.is_contiguous() and y.dtype == y1.dtype), "%s must be contiguous [%d, %d] in one dtype", name, T, H)
+    nxt = None
+    if next_gain is not None:
+        _f32(next_gain, (H,), "next_gain")
+        nxt = torch.empty((T, H), dtype=dtype, device=residual.device)
+    lib = build.load("gated_residual")
+    _check(lib.ga_gated_residual_add(_ptr(residual), _ptr(z), _ptr(y1), _ptr(y2), _i(T), _i(H), _i(_is_bf16(y1.dtype)),
+                                     _ptr(next_gain), _f(next_eps), _ptr(nxt), _i(_is_bf16(dtype) if nxt is not None else 0),
+                                     _stream()), "gated_residual_add")
+    return nxt

@@ -43,9 +43,20 @@ class PagedSpec:
     """Anything kept per token, in pages: `tensors` lists (name, elements per token) of every tensor a page holds; a
     page of the group's pool is, for each of them, page_size * elements in a row, which the mixer views as it likes.
     window: None keeps every token; an integer w keeps only what a token at position p can still see (positions > p - w).
-    Mixers with the same spec share a pool and a block table."""
+    Mixers with the same spec share a pool and a block table.
+    every: a row stands for this many consecutive positions (1: a row a token): row r belongs to the positions [r * every,
+    (r + 1) * every), a request of n tokens holds ceil(n / every) rows, and the step's slot mapping names, for every token,
+    the row of its block (what a mixer keeps per block of tokens: sums, means).  With every > 1 there is no window.
+    dtype: the number format of the pages; None: the model's."""
     tensors: Tuple[Tuple[str, int], ...]
     window: Optional[int] = None
+    every: int = 1
+    dtype: Optional[torch.dtype] = None
+
+    def __post_init__(self):
+        if int(self.every) < 1 or (int(self.every) > 1 and self.window is not None):
+            raise ValueError("a paged cache keeps a row per `every` >= 1 positions, and with every > 1 no window; got every "
+                             "%r, window %r" % (self.every, self.window))
 
     def page_tensors(self):
         return tuple((str(n), int(w)) for n, w in self.tensors)

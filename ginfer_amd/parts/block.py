@@ -197,3 +197,42 @@ def whole(delta, norm=None):
         total = delta.sum(dim=0)
         return total.to(norm.dtype) if norm is not None else total
     return delta
+
+
+@register_arrangement("parallel_gated")
+class ParallelGatedBlock(Arrangement):
+    """n = norm(x);  x <- x + (gate1(n) * mixer(n) + gate2(n) * feed_forward(n)): ONE norm, both sublayers read its rows side
+    by side, and each result enters the stream through a gate that reads the same rows (a part of the `residual_gate`
+    family: `logits(n)`, `add(residual, z, results, then)`).  A layer may have no feed-forward (its gate part then names one
+    gate).  The 32-bit stream is updated in place; where the model hands over the norm of the block that runs next
+    (`into_norm`), the launch that adds the results also makes that norm's rows (the next block then gets `NormedRows` in
+    place of a delta)."""
+
+    roles = {"norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward", "gate": "residual_gate"}
+    optional_roles = ("feed_forward",)
+
+    folds_output = True              # forward() takes `into_norm`
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.feed_forward = self._parts.get("feed_forward")
+        gates = len(getattr(self.gate, "names", ()))
+        if gates != (1 if self.feed_forward is None else 2):
+            raise ValueError("a block gates each of its sublayers: %d gates for %d sublayers"
+                             % (gates, 1 if self.feed_forward is None else 2))
+
+    def takes_folded_input(self):
+        """The norm whose rows this block takes ready-made (NormedRows) in place of a delta, or None."""
+        return self.norm if SandwichBlock._plain_gain(self.norm) else None
+
+    def forward(self, residual, delta, step, cache, into_norm=None):
+        if isinstance(delta, NormedRows):           # the block before has made this block's rows
+            n = delta.rows
+        else:
+            n = self.norm.forward(residual, whole(delta, self.norm))
+        z = self.gate.logits(n)
+        results = [self.mixer.forward(n, step, cache)]
+        if self.feed_forward is not None:
+            results.append(self.feed_forward.forward(n))
+        rows = self.gate.add(residual, z, [whole(r).to(n.dtype) if r.dim() == 3 else r for r in results], then=into_norm)
+        return NormedRows(rows) if into_norm is not None else None

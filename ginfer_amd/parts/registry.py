@@ -3,7 +3,7 @@ reaches it, so no part knows which model it is in.  New kinds register themselve
 decorators below; the model builder looks kinds up here and nowhere else."""
 
 _REGISTRIES = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "embedding": {}, "head": {},
-               "arrangement": {}, "convolution": {}, "reentry": {}}
+               "arrangement": {}, "convolution": {}, "reentry": {}, "residual_gate": {}}
 
 
 def _register(role, kind):
@@ -43,6 +43,10 @@ def register_convolution(kind):
 
 def register_reentry(kind):
     return _register("reentry", kind)
+
+
+def register_residual_gate(kind):
+    return _register("residual_gate", kind)
 
 
 def register_arrangement(kind):

@@ -73,3 +73,11 @@ class RotaryNeoX(Part):
             ang = p[:, None] * inv_freq[None, :]
             self._tables = (torch.cos(ang).to(self.device).contiguous(), torch.sin(ang).to(self.device).contiguous())
         return self._tables
+
+
+@register_position("rope_interleaved")
+class RotaryInterleaved(RotaryNeoX):
+    """The same angles and tables; the mixer's kernel turns the neighbouring coordinates (2j, 2j + 1) by angle j, where the
+    NeoX pairing turns (j, j + rotary_dim / 2)."""
+
+    style = "interleaved"
