@@ -92,6 +92,30 @@ def _potupel_size(width, ff, heads, kv_heads, layers=6, vocab=32768):
 POTUPEL_SIZES = {"1.5b": _potupel_size(1536, 8960, 12, 2), "7b": _potupel_size(3584, 18944, 28, 4)}
 
 
+# Layer sizes for the Puguzen design beside the Titozen design, the closest one the engine has (recurrent layers and windowed
+# attention, two to one), at equal width, feed-forward, heads, layers and vocabulary (--puguzen): gated linear attention,
+# retention and the attention over a window and pooled blocks in turn; the recurrent heads 64 x 128 as Titozen's, the
+# attention's heads 128 wide, the window as long as Titozen's, blocks of 64 tokens.
+def _puguzen_size(width, ff, heads, kv_heads, window, layers=6, vocab=32768):
+    mlp = dict(kind="dense", ff=ff)
+    gla = dict(type="gla", mixer=dict(heads=heads, dim=64, vdim=128, tau=16.0, rank=64), mlp=mlp)
+    ret = dict(type="retention", mlp=mlp, mixer=dict(heads=heads, dim=64, vdim=128, rot=dict(base=1e6, dims=64),
+                                                     decay=[1.0 - 2.0 ** (-5 - 4.0 * h / heads) for h in range(heads)]))
+    att = dict(type="attention", mlp=mlp, mixer=dict(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=0.1,
+                                                     mask=dict(size=window, pool=64), rot=dict(base=5e5, dims=64)))
+    puguzen = dict(architecture="Puguzen", vocab=vocab, width=width, norm=dict(eps=1e-5),
+                   layers=[(gla, ret, att)[i % 3] for i in range(layers)])
+    return puguzen
+
+
+PUGUZEN_SIZES = {"1.5b": (_puguzen_size(1536, 8960, 12, 2, 1024), TITOZEN_SIZES["1.5b"][0]),
+                 "7b": (_puguzen_size(3584, 18944, 28, 4, 2048), TITOZEN_SIZES["7b"][0])}
+
+
+def compare_puguzen(args):
+    return compare_designs(args, "puguzen", "Puguzen", args.puguzen, PUGUZEN_SIZES, beside=("titozen", "Titozen"))
+
+
 def compare_titozen(args):
     return compare_designs(args, "titozen", "Titozen", args.titozen, TITOZEN_SIZES)
 
@@ -100,7 +124,7 @@ def compare_potupel(args):
     return compare_designs(args, "potupel", "Potupel", args.potupel, POTUPEL_SIZES)
 
 
-def compare_designs(args, key, name, chosen, sizes):
+def compare_designs(args, key, name, chosen, sizes, beside=("qwen2", "Qwen2")):
     """Prefill of --prefill-tokens tokens and decode steps at --batch and the --points (contexts ending at --context)
     through Engine.step, for each size and each of the two designs."""
     import torch
@@ -109,14 +133,14 @@ def compare_designs(args, key, name, chosen, sizes):
     batches = sorted({int(p) for p in args.points.split(",") if p} | {args.batch})
     max_b = max(batches)
     g = torch.Generator().manual_seed(0)
-    out = {"metric": "prefill and decode tok/s of the %s design beside Qwen2 at equal sizes" % name, "unit": "tok/s", "n_gpus": 1,
+    out = {"metric": "prefill and decode tok/s of the %s design beside %s at equal sizes" % (name, beside[1]), "unit": "tok/s", "n_gpus": 1,
            "steps": args.steps, "warmup": args.warmup, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
            "data": "synthetic tokens, random weights", "prefill_tokens": T, "context": C, "sizes": {}}
     for size in [x for x in chosen.split(",") if x]:
         if size not in sizes:
             sys.exit("bench.py: --%s takes %s, got %r" % (key, ", ".join(sorted(sizes)), size))
         row = {}
-        for design, cfg in zip((key, "qwen2"), sizes[size]):
+        for design, cfg in zip((key, beside[0]), sizes[size]):
             engine = Engine(EngineConfig(
                 model_path=None, model_config=config_from_dict(cfg), random_seed=0, dtype=args.dtype,
                 max_num_batched_tokens=max(2048, T, C) + max_b, max_num_seqs=max_b, max_seq_len=max(T, C) + max_b + 24,
@@ -210,6 +234,9 @@ def main():
     ap.add_argument("--potupel", default=None, metavar="SIZES",
                     help="instead of the headline: the same comparison for the Potupel design (comma-separated: %s)"
                          % ", ".join(sorted(POTUPEL_SIZES)))
+    ap.add_argument("--puguzen", default=None, metavar="SIZES",
+                    help="instead of the headline: the same comparison for the Puguzen design (comma-separated: %s), beside "
+                         "the Titozen design at equal sizes" % ", ".join(sorted(PUGUZEN_SIZES)))
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on ONE GPU; --gpus %d is not supported" % args.gpus)
@@ -223,6 +250,9 @@ def main():
         return
     if args.potupel:
         print(json.dumps(compare_potupel(args)))
+        return
+    if args.puguzen:
+        print(json.dumps(compare_puguzen(args)))
         return
 
     shape_name, shape = SHAPES[args.shape]

@@ -133,36 +133,49 @@ def visible(i, T_keys, size, pool):
     return blocks, tokens
 
 
-def pooled_window_attention(n, w, p, m, eps, round_cache=None):
-    """round_cache: a function applied to keys and values before they are pooled and attended to (what a cache of
-    fewer bits does to them); None: nothing."""
-    T = n.shape[0]
-    H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    size, pool = m["mask"]["size"], m["mask"]["pool"]
-    q = (n @ w[p + "q"].T).view(T, H, D)
-    k = (n @ w[p + "k"].T).view(T, G, D)
-    v = (n @ w[p + "v"].T).view(T, G, V)
-    if m.get("rot"):
-        q, k = turn_neighbours(q, m["rot"]), turn_neighbours(k, m["rot"])
-    q, k = unit_rms(q, eps), unit_rms(k, eps)
-    if round_cache is not None:
-        k, v = round_cache(k), round_cache(v)
+def sigmoid_attention(q, k, v, bias, scale, size, pool):
+    """q [T, H, D], k [T, G, D], v [T, G, V] as the cache holds them, bias [H]: every token over its window and the means
+    of the blocks before it, weights sigmoid(scale q . k + bias), not normalised.  Returns [T, H, V]."""
+    T, H = q.shape[0], q.shape[1]
+    G = k.shape[1]
     nblocks = T // pool
     kp = torch.stack([k[b * pool:(b + 1) * pool].mean(dim=0) for b in range(nblocks)]) if nblocks else k[:0]
     vp = torch.stack([v[b * pool:(b + 1) * pool].mean(dim=0) for b in range(nblocks)]) if nblocks else v[:0]
-    out = torch.zeros((T, H, V), dtype=n.dtype)
+    out = torch.zeros((T, H, v.shape[2]), dtype=q.dtype)
     per = H // G
     for i in range(T):
         blocks, tokens = visible(i, T, size, pool)
         blocks = [b for b in blocks if b < nblocks]
         keys = torch.cat([kp[blocks], k[tokens]]) if blocks else k[tokens]
         vals = torch.cat([vp[blocks], v[tokens]]) if blocks else v[tokens]
-        for h in range(H):
-            g = h // per
-            s = (keys[:, g] @ q[i, h]) * float(m["scale"]) + w[p + "pb"][h]
-            out[i, h] = torch.sigmoid(s) @ vals[:, g]
+        group = [h // per for h in range(H)]             # query head h reads kv head h // (H / G)
+        s = torch.einsum("nhd,hd->nh", keys[:, group], q[i]) * float(scale) + bias
+        out[i] = torch.einsum("nh,nhv->hv", torch.sigmoid(s), vals[:, group])
+    return out
+
+
+def attention_inputs(n, w, p, m, eps, first_position=0):
+    """(q [T, H, D], k [T, G, D], v [T, G, V]) behind projection, rotation and the unit norm."""
+    T = n.shape[0]
+    H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    q = (n @ w[p + "q"].T).view(T, H, D)
+    k = (n @ w[p + "k"].T).view(T, G, D)
+    v = (n @ w[p + "v"].T).view(T, G, V)
+    if m.get("rot"):
+        q, k = turn_neighbours(q, m["rot"], first_position), turn_neighbours(k, m["rot"], first_position)
+    return unit_rms(q, eps), unit_rms(k, eps), v
+
+
+def pooled_window_attention(n, w, p, m, eps, round_cache=None):
+    """round_cache: a function applied to keys and values before they are pooled and attended to (what a cache of
+    fewer bits does to them); None: nothing."""
+    T = n.shape[0]
+    q, k, v = attention_inputs(n, w, p, m, eps)
+    if round_cache is not None:
+        k, v = round_cache(k), round_cache(v)
+    out = sigmoid_attention(q, k, v, w[p + "pb"], m["scale"], m["mask"]["size"], m["mask"]["pool"])
     gate = torch.sigmoid(n @ w[p + "g"].T)
-    return (out.reshape(T, H * V) * gate) @ w[p + "o"].T
+    return (out.reshape(T, -1) * gate) @ w[p + "o"].T
 
 
 def relu_glu(n, w, p):
@@ -191,3 +204,13 @@ def forward(cfg, w, ids, streams=None, **kw):
         if streams is not None:
             streams.append(x.clone())
     return centered_norm(x, w["final.norm"], eps) @ w["embed"].T
+
+
+def logits(ids, w, cfg):
+    return forward(cfg, w, ids)
+
+
+def residual_streams(ids, w, cfg):
+    streams = []
+    forward(cfg, w, ids, streams)
+    return torch.stack(streams)

@@ -1,0 +1,770 @@
+"""The Puguzen decoder in the engine against its plain statement (plain_puguzen.py), on the GPU: each mechanism alone,
+then whole models under every way of cutting and batching, in 32-bit and in bfloat16, at sizes of the tests' own."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import plain_puguzen as pp
+from test_puguzen import GLA, RET, ATT, config
+
+pytestmark = pytest.mark.gpu
+
+# Sizes that differ from one another wherever the design allows it: keys wider and narrower than values and as wide; one
+# kv head for all, one per head, groups; the rotation on a part of a head, on all of it and absent; windows of 1 to 33
+# tokens, blocks of 1 to 16, blocks longer than the window; tau 1 to 16, ranks 1 to 7; layers without a feed-forward; every
+# order of the three mixers.
+MIX = config(96, 211, [
+    (ATT(4, 2, 12, 20, 0.4, 9, 4, rot=(100.0, 8)), 136),
+    (GLA(3, 8, 12, 4.0, rank=5), None),
+    (RET(2, 16, 8, (0.9, 0.995), rot=(50.0, 6)), 40),
+    (ATT(3, 3, 8, 8, 0.3, 5, 7), 24),
+    (GLA(1, 24, 16, 1.0, rank=1), 32),
+], eps=2e-6)
+WIDE = config(64, 150, [
+    (RET(5, 12, 20, (0.5, 0.8, 0.9, 0.97, 1.0)), 72),
+    (ATT(6, 1, 16, 24, 0.25, 33, 16, rot=(1e4, 16)), 64),
+    (GLA(2, 40, 8, 16.0, rank=7), None),
+], eps=1e-5)
+TINY = config(40, 64, [(ATT(1, 1, 16, 16, 0.5, 1, 1, rot=(50.0, 2)), 8)])
+DEEP = config(48, 97, [
+    (GLA(4, 4, 4, 2.0, rank=3), 40),
+    (RET(1, 32, 48, (0.97,), rot=(777.0, 32)), None),
+    (ATT(8, 4, 8, 12, 0.35, 20, 3), 20),
+    (ATT(2, 2, 24, 8, 0.2, 6, 10, rot=(10.0, 24)), None),
+], eps=1e-4)
+CONFIGS = {"mix": (MIX, 8), "wide": (WIDE, 16), "tiny": (TINY, 16), "deep": (DEEP, 32)}
+STD = 5.0
+
+
+def make_folder(path, cfg, seed, std_scale=STD, edit=None):
+    """A model folder with random weights, stored in bfloat16 as this design's checkpoints are (so the 32-bit engine, the
+    bfloat16 engine and the plain statement all start from the same numbers); `edit(tensors)` may change them before
+    they are written."""
+    folder = H.make_model_folder(path, cfg, seed, "bfloat16", std_scale=std_scale)
+    from safetensors.torch import load_file, save_file
+    file = os.path.join(folder, "model.safetensors")
+    tensors = {k: v.clone() for k, v in load_file(file).items()}
+    (edit or sharpen)(tensors)
+    save_file(tensors, file)
+    return folder
+
+
+def sharpen(tensors, std_scale=STD):
+    """Biases and the decay's widening keep the spread their specs name (the folder's wider draw would push every sigmoid
+    to 0 or 1); the attention's biases sit below zero, so that few keys carry a row and one that is wrongly seen or missed
+    moves it."""
+    for name, t in tensors.items():
+        if name.endswith((".rg1.b", ".rg2.b", ".a2.b", ".a2")):
+            t /= std_scale
+        if name.endswith(".mix.pb"):
+            t.copy_((t / std_scale - 1.5).to(t.dtype))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {name: make_folder(tmp_path_factory.mktemp(name), cfg, seed=i) for i, (name, (cfg, _)) in enumerate(CONFIGS.items())}
+
+
+def runner_for(folder, name, dtype, tokens=1024, max_requests=4, **kw):
+    from ginfer_amd import ModelRunner
+    ps = CONFIGS[name][1]
+    return ModelRunner(folder, dtype=dtype, page_size=ps, num_pages=-(-tokens // ps), max_requests=max_requests,
+                       max_model_len=2048, **kw)
+
+
+def requests_for(name, lengths, seed=20):
+    return {"q%d" % i: H.random_tokens(n, CONFIGS[name][0]["vocab"], seed + i) for i, n in enumerate(lengths)}
+
+
+_plain = {}
+
+
+def plain(folder, ids):
+    key = (folder, tuple(ids))
+    if key not in _plain:
+        _plain[key] = pp.logits(ids, pp.read_weights(folder), pp.read_config(folder)).numpy()
+    return _plain[key]
+
+
+def compare(got, requests, folder, tol, what, close_calls=0.0, median=0.5):
+    """Every row against the plain statement.  close_calls: the share of rows that may miss the tolerance."""
+    over, first, errors = 0, None, []
+    for (rid, p), row in sorted(got.items()):
+        ref = plain(folder, requests[rid])
+        assert np.isfinite(row).all(), "%s: request %s position %d: non-finite logits" % (what, rid, p)
+        err = float(np.abs(row.astype(np.float64) - ref[p]).max() / np.abs(ref).max())
+        errors.append(err)
+        if err > tol:
+            over += 1
+            first = first or "%s: first wrong place is request %s position %d of %d: error %.3g > %.3g" % (
+                what, rid, p, len(requests[rid]), err, tol)
+    assert over <= close_calls * len(got), "%s (%d of %d rows)" % (first, over, len(got))
+    assert float(np.median(errors)) <= tol * median, "%s: the median row is off by %.3g" % (what, float(np.median(errors)))
+    for rid, ids in requests.items():
+        missing = [p for p in range(len(ids)) if (rid, p) not in got]
+        assert not missing, "%s: request %s lacks logits at %s" % (what, rid, missing[:8])
+
+
+# 32-bit differs from the 64-bit plain statement by the rounding of sums of a few hundred terms; bfloat16 rounds every stored
+# activation to 8 bits: the median row must stay within half the tolerance and a few rows may miss it
+TOL = {"float32": 1e-4, "bfloat16": 6e-2}
+CLOSE = {"float32": 0.0, "bfloat16": 0.05}
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+class _Step:
+    """The few arrays of a step that the kernels under test read."""
+
+    def __init__(self, q_len, q_start):
+        dev = torch.device("cuda")
+        cu = np.concatenate([[0], np.cumsum(q_len)]).astype(np.int32)
+        self.cu_tokens = torch.tensor(cu, device=dev)
+        self.q_start = torch.tensor(q_start, dtype=torch.int32, device=dev)
+        self.token_entry = torch.tensor(np.repeat(np.arange(len(q_len)), q_len), dtype=torch.int32, device=dev)
+        self.positions = torch.tensor(np.concatenate([np.arange(s, s + n) for s, n in zip(q_start, q_len)]), dtype=torch.int32,
+                                      device=dev)
+        self.num_entries = len(q_len)
+        self.host_q_len, self.host_q_start = list(q_len), list(q_start)
+        self.extra = {}
+
+    @property
+    def max_q_len(self):
+        return max(self.host_q_len)
+
+    @property
+    def max_kv_len(self):
+        return max(s + n for s, n in zip(self.host_q_start, self.host_q_len))
+
+
+# ----------------------------------------------------------------------------------------------- mechanisms alone
+
+def test_gated_sum_into_the_stream_and_the_next_norm():
+    from ginfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(0)
+    sig = torch.sigmoid
+    for width in (7, 96, 328, 1000, 4100):
+        res = torch.randn((5, width), generator=g) * 3
+        z = torch.randn((5, 2 * width), generator=g) * 2
+        nxt = torch.randn((width,), generator=g)
+        for dtype, tol in ((torch.float32, 2e-6), (torch.bfloat16, 1e-2)):
+            y1, y2 = (torch.randn((5, width), generator=g).to(dtype) for _ in range(2))
+            want2 = res.double() + (sig(z[:, :width].double()) * y1.double() + sig(z[:, width:].double()) * y2.double())
+            want1 = res.double() + sig(z[:, :width].double()) * y1.double()
+            r = res.cuda().clone()
+            rows = ops.gated_residual_add(r, z.cuda(), y1.cuda(), y2.cuda(), next_gain=nxt.cuda(), next_eps=3e-6, dtype=dtype)
+            assert H.rel_err(r.cpu(), want2) < 2e-6
+            assert H.rel_err(rows.float().cpu(), pp.centered_norm(want2, nxt.double() - 1.0, 3e-6)) < tol
+            r2 = res.cuda().clone()
+            assert ops.gated_residual_add(r2, z.cuda(), y1.cuda(), y2.cuda()) is None and torch.equal(r2, r)
+            r1 = res.cuda().clone()
+            ops.gated_residual_add(r1, z[:, :width].contiguous().cuda(), y1.cuda())
+            assert H.rel_err(r1.cpu(), want1) < 2e-6
+
+
+def test_relu_as_the_limit_of_the_bounded_gate():
+    """relu(gate) * up from the gated activation with no bound, a step in place of the sigmoid and no shift: its own
+    pass over a product, and the epilogue of the weight-streaming product (few rows, bfloat16)."""
+    from ginfer_amd.kernels import ops
+    from ginfer_amd.parts.mlp import ClampedGLU
+    g = torch.Generator().manual_seed(1)
+    inf = float("inf")
+    for inter in (24, 37):
+        gu = torch.randn((9, 2 * inter), generator=g)
+        gu[0, :3] = 0.0
+        gu[1, 0] = -0.0
+        for dtype in (torch.float32, torch.bfloat16):
+            x = gu.to(dtype)
+            got = ops.clamped_glu(x.cuda(), inf, inf, 0.0).float().cpu()
+            want = (torch.relu(x[:, :inter].float()) * x[:, inter:].float()).to(dtype).float()
+            assert torch.equal(got, want)
+    W, I = 64, 48
+    w = {n: (torch.randn(s, generator=g) * 0.3).to(torch.bfloat16) for n, s in (("gate", (I, W)), ("up", (I, W)), ("down", (W, I)))}
+    ref = lambda x: pp.relu_glu(x.double(), {"m." + n: t.double() for n, t in w.items()}, "m.")
+    for dtype, tol in ((torch.float32, 2e-6), (torch.bfloat16, 2e-2)):
+        part = ClampedGLU(W, I, inf, dtype, "cuda", alpha=inf, shift=0.0)
+        part.bind_weights({n: t.cuda().to(dtype) for n, t in w.items()})
+        for rows in (1, 5, 16, 70):
+            x = torch.randn((rows, W), generator=g).to(torch.bfloat16)
+            assert H.rel_err(part.forward(x.cuda().to(dtype)).float().cpu(), ref(x)) < tol, (dtype, rows)
+
+
+def test_decay_of_gated_linear_attention():
+    from ginfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(2)
+    for channels, rank, tau, tokens in ((24, 5, 4.0, 7), (64, 16, 16.0, 3), (5, 1, 1.0, 2), (300, 7, 2.5, 4)):
+        proj = torch.randn((tokens, 11 + rank), generator=g)
+        a2, b = torch.randn((channels, rank), generator=g) * 3, torch.randn((channels,), generator=g) * 3
+        b[0], b[1 % channels] = 60.0, -60.0            # far out on both sides
+        got = ops.gla_decay(proj.cuda(), 11, a2.cuda(), b.cuda(), tau).cpu()
+        z = proj[:, 11:].double() @ a2.double().T + b.double()
+        want = torch.exp(torch.nn.functional.logsigmoid(z) / tau)
+        assert torch.isfinite(got).all() and float((got.double() - want).abs().max()) < 2e-6
+
+
+def _scan_case(seed, heads, dim, vdim, T, rot=None):
+    g = torch.Generator().manual_seed(seed)
+    width = 2 * heads * dim + heads * vdim + 3
+    proj = torch.randn((T, width), generator=g)
+    decay = torch.rand((T, heads * dim), generator=g) * 0.5 + 0.5
+    return proj, decay
+
+
+@pytest.mark.parametrize("heads, dim, vdim", [(2, 32, 32), (3, 8, 12), (1, 100, 20), (2, 256, 24), (5, 16, 64), (1, 1, 1)])
+def test_recurrence_across_cuts_and_a_slot_that_was_used(heads, dim, vdim):
+    """Both kinds of decay (per token and channel; per head, with rotated q and k), a whole sequence in one call against
+    the plain recurrence, then cut into calls of 1 to 40 tokens beside a second request, through slots that hold what
+    other requests left: the same bits."""
+    from ginfer_amd.kernels import ops
+    T = 90
+    proj, decay = _scan_case(heads * 1000 + dim, heads, dim, vdim, T)
+    k0, v0 = heads * dim, 2 * heads * dim
+    q = proj[:, :k0].double().view(T, heads, dim)
+    k = proj[:, k0:v0].double().view(T, heads, dim)
+    v = proj[:, v0:v0 + heads * vdim].double().view(T, heads, vdim)
+    r = dim - dim % 2 if dim > 1 else 0
+    rot = dict(base=30.0, dims=min(r, 6)) if r else None
+    hd = torch.linspace(0.6, 1.0, heads)
+    cases = [("channel", dict(decay=decay.cuda(), q_scale=dim ** -0.5),
+              pp.decayed_outer_recurrence(q / math.sqrt(dim), k, v, decay.double().view(T, heads, dim)))]
+    if rot:
+        a = pp.angles(rot, range(256))
+        tables = dict(cos=torch.cos(a).float().cuda().contiguous(), sin=torch.sin(a).float().cuda().contiguous())
+        cases.append(("head", dict(head_decay=hd.cuda(), k_scale=dim ** -0.5, **tables),
+                      pp.decayed_outer_recurrence(pp.turn_halves(q, rot), pp.turn_halves(k, rot) / math.sqrt(dim), v,
+                                                  hd.double()[None, :, None].expand(T, heads, dim))))
+    else:
+        cases.append(("head", dict(head_decay=hd.cuda()),
+                      pp.decayed_outer_recurrence(q, k, v, hd.double()[None, :, None].expand(T, heads, dim))))
+    for kind, kw, want in cases:
+        state = torch.full((4, heads, dim, vdim), 1e4, dtype=torch.float32, device="cuda")
+        slots = torch.tensor([2], dtype=torch.int64, device="cuda")
+        whole = ops.decay_scan(proj.cuda(), 0, k0, v0, state, slots, _Step([T], [0]), heads, dim, vdim, **kw).cpu()
+        assert H.rel_err(whole, want) < 1e-5, kind
+        final = state[2].clone()
+        # cut, beside another request whose tokens come first in the step
+        state.fill_(-3e3)
+        other = torch.randn((7, proj.shape[1]), generator=torch.Generator().manual_seed(5))
+        got, at = [], 0
+        for n in [1, 1, 2, 16, 17, 40, 1, 3, 9]:
+            both = torch.cat([other, proj[at:at + n]]).cuda()
+            step = _Step([7, n], [at + 3, at])
+            kw2 = dict(kw)
+            if "decay" in kw2:
+                kw2["decay"] = torch.cat([torch.full((7, heads * dim), 0.5), decay[at:at + n]]).cuda()
+            out = ops.decay_scan(both, 0, k0, v0, state, torch.tensor([0, 3], dtype=torch.int64, device="cuda"), step, heads,
+                                 dim, vdim, **kw2)
+            got.append(out[7:].cpu())
+            at += n
+        assert at == T and torch.equal(torch.cat(got), whole), kind
+        assert torch.equal(state[3], final), kind
+
+
+def test_heads_normed_and_gated():
+    from ginfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(3)
+    for heads, vdim in ((2, 32), (3, 12), (1, 200), (5, 1)):
+        x = torch.randn((6, heads, vdim), generator=g) * 4
+        w = torch.randn((vdim,), generator=g)
+        proj = torch.randn((6, 9 + heads * vdim), generator=g) * 2
+        gate = proj[:, 9:].double()
+        silu = (gate * torch.sigmoid(gate)).view(6, heads, vdim)
+        for dtype, tol in ((torch.float32, 2e-6), (torch.bfloat16, 1e-2)):
+            got = ops.head_norm_gate(x.cuda(), w.cuda(), 1e-5, dtype, proj=proj.cuda(), gate_start=9).float().cpu()
+            assert H.rel_err(got, (pp.unit_rms(x.double(), 1e-5) * w.double() * silu).reshape(6, -1)) < tol
+            got = ops.head_norm_gate(x.cuda(), None, 1e-5, dtype).float().cpu()
+            assert H.rel_err(got, pp.unit_rms(x.double(), 1e-5).reshape(6, -1)) < tol
+
+
+class _AttentionCase:
+    """Pages of tokens and of blocks made by hand (the pages in no order), and a sequence run through the three kernels in
+    cuts of the caller's choice."""
+
+    def __init__(self, nh, nkv, dim, vdim, size, pool, page, dtype, T, pages=None):
+        self.nh, self.nkv, self.dim, self.vdim, self.size, self.pool, self.page, self.dtype = nh, nkv, dim, vdim, size, pool, page, dtype
+        n = pages or -(-T // page) + 2
+        self.k_rows = torch.full((n, page * nkv * dim), 9e3, dtype=dtype, device="cuda")      # what other requests left
+        self.v_rows = torch.full((n, page * nkv * vdim), 9e3, dtype=dtype, device="cuda")
+        self.pk = torch.full((n, page * nkv * dim), 9e3, dtype=torch.float32, device="cuda")
+        self.pv = torch.full((n, page * nkv * vdim), 9e3, dtype=torch.float32, device="cuda")
+        rng = np.random.RandomState(T + page)
+        self.table = torch.tensor(rng.permutation(n)[None, :].astype(np.int32), device="cuda")
+        self.pool_table = torch.tensor(rng.permutation(n)[None, :].astype(np.int32), device="cuda")
+
+    def slots(self, table, rows):
+        t = table[0].cpu().numpy()
+        return torch.tensor([int(t[r // self.page]) * self.page + r % self.page for r in rows], dtype=torch.int64, device="cuda")
+
+    def run(self, proj, cuts, bias, scale, cos=None, sin=None, unit=False, gate_start=None, eps=1e-6):
+        from ginfer_amd.kernels import ops
+        out, at = [], 0
+        for n in cuts:
+            step = _Step([n], [at])
+            rows = range(at, at + n)
+            p = proj[at:at + n].cuda()
+            q = ops.pooled_attention_prepare(p, step.positions, cos, sin, self.slots(self.table, rows), self.k_rows, self.v_rows,
+                                             self.nh, self.nkv, self.dim, self.vdim, eps, unit_norm=unit)
+            ops.pooled_attention_pool(self.pk, self.pv, self.k_rows, self.v_rows, step, self.table,
+                                      self.slots(self.pool_table, [r // self.pool for r in rows]), self.nkv, self.dim, self.vdim,
+                                      self.pool, self.page)
+            out.append(ops.pooled_attention(q, self.k_rows, self.v_rows, self.pk, self.pv, step, self.table, self.pool_table,
+                                            bias, self.nh, self.nkv, self.dim, self.vdim, self.size, self.pool, self.page, scale,
+                                            self.dtype, proj=p if gate_start is not None else None,
+                                            gate_start=gate_start or 0).float().cpu())
+            at += n
+        assert at == proj.shape[0]
+        return torch.cat(out)
+
+
+def _split(proj, nh, nkv, dim, vdim, dtype):
+    """q, k, v of a projection as the kernels hold them: q in 32-bit, k and v rounded as the cache rounds them."""
+    T = proj.shape[0]
+    a, b = nh * dim, (nh + nkv) * dim
+    q = proj[:, :a].double().view(T, nh, dim)
+    k = proj[:, a:b].to(dtype).double().view(T, nkv, dim)
+    v = proj[:, b:b + nkv * vdim].to(dtype).double().view(T, nkv, vdim)
+    return q, k, v
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh, nkv, dim, vdim, size, pool, page", [
+    (4, 2, 16, 16, 37, 11, 16), (3, 3, 12, 20, 9, 4, 8), (6, 1, 24, 8, 5, 7, 16), (2, 2, 64, 64, 70, 64, 32),
+    (1, 1, 8, 8, 1, 1, 8), (8, 4, 40, 136, 130, 3, 16)])
+def test_attention_over_window_and_blocks_whole_and_cut(nh, nkv, dim, vdim, size, pool, page, dtype):
+    """Random keys, a bias per head, the gate: a sequence of several windows at once against the plain mechanism, then in
+    cuts down to single tokens and pairs (in 32-bit: the same bits)."""
+    dt = DT[dtype]
+    T = min(3 * size + 2 * pool + 11, 330)
+    g = torch.Generator().manual_seed(size * 100 + pool)
+    proj = torch.randn((T, (nh + nkv) * dim + nkv * vdim + nh * vdim), generator=g)
+    bias = torch.randn((nh,), generator=g) - 1.0
+    q, k, v = _split(proj, nh, nkv, dim, vdim, dt)
+    gate0 = (nh + nkv) * dim + nkv * vdim
+    want = pp.sigmoid_attention(q, k, v, bias.double(), 0.3, size, pool) * torch.sigmoid(proj[:, gate0:].double()).view(T, nh, vdim)
+    tol = 1e-5 if dtype == "float32" else 1e-2
+    outs = []
+    for cuts in ([T], [b - a for a, b in H.cut(T, (1, 2, 1, 5, 33, 2, 64, 3))], [1] * T):
+        case = _AttentionCase(nh, nkv, dim, vdim, size, pool, page, dt, T)
+        outs.append(case.run(proj, cuts, bias.cuda(), 0.3, gate_start=gate0))
+        assert H.rel_err(outs[-1], want.reshape(T, -1)) < tol, cuts[:4]
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("how", ["whole", "decoded"])
+def test_one_key_made_to_stand_out(dtype, how):
+    """Every weight is near zero but one: the query of the last token matches one earlier token, whose value is marked.
+    Where that token is decides what comes out: inside the window its value; in a block that is seen, a share 1 / pool of
+    it at the block's weight; behind the window in a block that is not seen yet, nothing.  At page borders, at the first
+    tokens, far back."""
+    dt = DT[dtype]
+    nh, nkv, dim, vdim, size, pool, page = 2, 1, 16, 8, 20, 6, 16
+    T = 200
+    last = T - 1
+    lo = last - size + 1                              # first token of the window: 180; blocks 0..29 end before it (30 * 6 = 180)
+    places = {"window_first": lo, "window_last": last, "just_outside_in_a_seen_block": lo - 1, "far_block": 7, "first_token": 0,
+              "page_border": 16 * 5, "before_page_border": 16 * 5 - 1, "block_first": 6 * 20, "block_last": 6 * 20 + 5}
+    # a second geometry where the window's edge cuts a block: size 21 -> lo = 179, block 29 (174..179) not seen, 174..178 unseen
+    for name, (sz, place, seen) in dict(
+            {n: (size, p, "token" if p >= lo else "block") for n, p in places.items()},
+            unseen_behind_the_window=(21, 176, None), first_of_the_window_in_an_unseen_block=(21, 179, "token"),
+            last_seen_block=(21, 173, "block")).items():
+        g = torch.Generator().manual_seed(11)
+        proj = torch.randn((T, (nh + nkv) * dim + nkv * vdim), generator=g) * 0.05
+        a, b = nh * dim, (nh + nkv) * dim
+        proj[last, :a] = 0.0
+        proj[last, 0] = proj[last, dim] = 6.0          # both heads' queries read coordinate 0
+        proj[place, a] = 6.0 * (pool if seen == "block" else 1)     # the key; a block's mean keeps a pool-th of it
+        proj[:, b:] = 0.01
+        proj[place, b:] = 7.0
+        bias = torch.full((nh,), -9.0)
+        q, k, v = _split(proj, nh, nkv, dim, vdim, dt)
+        want = pp.sigmoid_attention(q, k, v, bias.double(), 1.0, sz, pool)[last]
+        case = _AttentionCase(nh, nkv, dim, vdim, sz, pool, page, dt, T)
+        cuts = [T] if how == "whole" else [T - 30] + [1] * 30
+        got = case.run(proj, cuts, bias.cuda(), 1.0)[last].view(nh, vdim)
+        assert H.rel_err(got, want) < (1e-5 if dtype == "float32" else 1e-2), name
+        expect = {"token": 7.0, "block": 7.0 / pool, None: 0.0}[seen]
+        assert abs(float(got.mean()) - expect) < 0.15, (name, float(got.mean()), expect)
+
+
+def test_rotation_of_neighbours_and_unit_norm_before_the_cache():
+    from ginfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(4)
+    for nh, nkv, dim, vdim, dims in ((4, 2, 16, 12, 16), (3, 1, 24, 8, 6), (2, 2, 200, 5, 64), (1, 1, 7, 3, 0)):
+        T, first = 9, 37
+        proj = torch.randn((T, (nh + nkv) * dim + nkv * vdim + 5), generator=g) * 3
+        rot = dict(base=200.0, dims=dims) if dims else None
+        cos = sin = None
+        if rot:
+            a = pp.angles(rot, range(64))
+            cos, sin = torch.cos(a).float().cuda().contiguous(), torch.sin(a).float().cuda().contiguous()
+        q = proj[:, :nh * dim].double().view(T, nh, dim)
+        k = proj[:, nh * dim:(nh + nkv) * dim].double().view(T, nkv, dim)
+        if rot:
+            q, k = pp.turn_neighbours(q, rot, first), pp.turn_neighbours(k, rot, first)
+        q, k = pp.unit_rms(q, 1e-5), pp.unit_rms(k, 1e-5)
+        v = proj[:, (nh + nkv) * dim:(nh + nkv) * dim + nkv * vdim].double()
+        for dt, tol in ((torch.float32, 2e-6), (torch.bfloat16, 1e-2)):
+            k_rows = torch.zeros((40, nkv * dim), dtype=dt, device="cuda")
+            v_rows = torch.zeros((40, nkv * vdim), dtype=dt, device="cuda")
+            slots = torch.tensor([31, 2, 5, 39, 0, -1, 7, 8, 9], dtype=torch.int64, device="cuda")
+            positions = torch.arange(first, first + T, dtype=torch.int32, device="cuda")
+            got = ops.pooled_attention_prepare(proj.cuda(), positions, cos, sin, slots, k_rows, v_rows, nh, nkv, dim, vdim, 1e-5)
+            assert H.rel_err(got.cpu(), q.reshape(T, -1)) < 2e-6
+            keep = [i for i, s in enumerate(slots.tolist()) if s >= 0]
+            rows = [slots[i].item() for i in keep]
+            assert H.rel_err(k_rows[rows].float().cpu(), k.reshape(T, -1)[keep]) < tol
+            assert H.rel_err(v_rows[rows].float().cpu(), v[keep]) < tol
+            untouched = [r for r in range(40) if r not in rows]
+            assert float(k_rows[untouched].abs().max()) == 0.0          # a token without a slot writes nothing
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixers_alone_whole_against_cut(dtype):
+    """Each mixer part by itself, driven with hand-made caches: a whole sequence in one step against the plain
+    mechanism, then the same sequence in cuts, through state that another request left."""
+    from ginfer_amd.parts.linear_attention import GatedLinearAttention, Retention
+    from ginfer_amd.parts.pooled_attention import PooledWindowAttention
+    from ginfer_amd.parts.rope import RotaryNeoX, RotaryInterleaved
+    from ginfer_amd.parts.model import KVView, StateView
+    dt = DT[dtype]
+    g = torch.Generator().manual_seed(7)
+    W, T, eps = 40, 61, 1e-5
+    x = torch.randn((T, W), generator=g).to(torch.bfloat16)
+    tol = 2e-5 if dtype == "float32" else 3e-2
+
+    def weights(shapes):
+        return {n: (torch.randn(s, generator=g) * (1.0 if n in ("pb", "a2.b", "a2", "norm") else 0.3)).to(torch.bfloat16)
+                for n, s in shapes.items()}
+
+    def run_state(part, cuts):
+        state = torch.full((3,) + tuple(part.cache_spec().shape), 1e4, dtype=torch.float32, device="cuda")
+        got, at = [], 0
+        for n in cuts:
+            sv = StateView(state, torch.tensor([1], dtype=torch.int64, device="cuda"), True)
+            got.append(part.forward(x[at:at + n].cuda().to(dt), _Step([n], [at]), sv).float().cpu())
+            at += n
+        return torch.cat(got)
+    cuts = [1, 1, 2, 5, 3, 16, 1, 31, 1]
+    m = dict(heads=3, dim=8, vdim=12, tau=4.0)
+    w = weights({"q": (24, W), "k": (24, W), "v": (36, W), "g": (36, W), "o": (W, 36), "norm": (12,), "a1": (5, W), "a2": (24, 5), "a2.b": (24,)})
+    part = GatedLinearAttention(W, 3, 8, 12, 5, 4.0, eps, dt, "cuda")
+    part.bind_weights({n: t.cuda().to(dt) for n, t in w.items()})
+    ref = pp.gla(x.double(), {"m." + n: t.double() for n, t in w.items()}, "m.", m, eps)
+    for c in ([T], cuts):
+        assert H.rel_err(run_state(part, c), ref) < tol, ("gla", c)
+    m = dict(heads=2, dim=16, vdim=8, decay=[0.9, 0.99], rot=dict(base=50.0, dims=6))
+    w = weights({"q": (32, W), "k": (32, W), "v": (16, W), "g": (16, W), "o": (W, 16)})
+    part = Retention(W, 2, 16, 8, (0.9, 0.99), eps, dt, "cuda", position=RotaryNeoX(50.0, 6, 128, device="cuda", wide_frequencies=True))
+    part.bind_weights({n: t.cuda().to(dt) for n, t in w.items()})
+    ref = pp.retention(x.double(), {"m." + n: t.double() for n, t in w.items()}, "m.", m, eps)
+    for c in ([T], cuts):
+        assert H.rel_err(run_state(part, c), ref) < tol, ("retention", c)
+    m = dict(heads=4, kv_heads=2, dim=12, vdim=20, scale=0.4, mask=dict(size=9, pool=4), rot=dict(base=100.0, dims=8))
+    w = weights({"q": (48, W), "k": (24, W), "v": (40, W), "g": (80, W), "o": (W, 80), "pb": (4,)})
+    part = PooledWindowAttention(W, 4, 2, 12, 20, 0.4, 9, 4, eps, dt, "cuda",
+                                 position=RotaryInterleaved(100.0, 8, 128, device="cuda", wide_frequencies=True))
+    part.bind_weights({n: t.cuda().to(dt) for n, t in w.items()})
+    rounded = (lambda t: t.to(dt).double())
+    ref = pp.pooled_window_attention(x.double(), {"m." + n: t.double() for n, t in w.items()}, "m.", m, eps, round_cache=rounded)
+    ps, pages = 8, 10
+    for c in ([T], cuts):
+        store = {n: torch.full((pages, ps * width), 9e3, dtype=d, device="cuda")
+                 for n, width, d in (("k", 24, dt), ("v", 40, dt), ("pk", 24, torch.float32), ("pv", 40, torch.float32))}
+        table = torch.tensor([[7, 2, 9, 0, 4, 1, 8, 3]], dtype=torch.int32, device="cuda")
+        ptable = torch.tensor([[5, 6, 0, 3, 1, 2, 4, 7]], dtype=torch.int32, device="cuda")
+        got, at = [], 0
+        for n in c:
+            slot = lambda t, rows: torch.tensor([int(t[0, r // ps]) * ps + r % ps for r in rows], dtype=torch.int64, device="cuda")
+            near = KVView(None, None, table, slot(table, range(at, at + n)), ps, True, pages=dict(k=store["k"], v=store["v"]))
+            means = KVView(None, None, ptable, slot(ptable, [p // 4 for p in range(at, at + n)]), ps, True,
+                           pages=dict(k=store["pk"], v=store["pv"]))
+            got.append(part.forward(x[at:at + n].cuda().to(dt), _Step([n], [at]), [near, means]).float().cpu())
+            at += n
+        assert H.rel_err(torch.cat(got), ref) < tol, ("attention", c)
+
+
+# ----------------------------------------------------------------------------------------------- whole models
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_decoded_and_in_portions(folders, name, dtype):
+    """Every request whole; then most of it in one step and the rest token by token; then in portions of 1 to 64
+    tokens, and in pairs.  In 32-bit the four agree to the bit."""
+    reqs = requests_for(name, [1, 2, 5, 44, 131])
+    runner = runner_for(folders[name], name, dtype)
+    got = {}
+    for what, steps in (("whole", H.steps_whole(reqs)), ("decoded", H.steps_last_decoded(reqs, last=48)),
+                        ("portions", H.steps_portions(reqs)), ("pairs", H.steps_portions(reqs, sizes=(2,)))):
+        got[what] = H.run_steps(runner, steps)
+        runner.cache.check()
+        compare(got[what], reqs, folders[name], TOL[dtype], "%s %s %s" % (name, dtype, what), CLOSE[dtype])
+    if dtype == "float32":
+        for what in ("decoded", "portions", "pairs"):
+            for key, row in got["whole"].items():
+                assert np.array_equal(row, got[what][key]), "%s: %s differs from whole at %s" % (name, what, key)
+    assert not runner.cache.requests and all(g.pool.num_free == g.pool.num_pages for g in runner.cache.groups)
+
+
+def test_the_stream_after_every_layer(folders):
+    name = "mix"
+    ids = H.random_tokens(37, CONFIGS[name][0]["vocab"], 5)
+    runner = runner_for(folders[name], name, "float32", use_graphs=False)
+    seen = []
+    for block in runner.model.blocks:
+        def wrapped(residual, delta, step, cache, inner=block.forward, **kw):
+            out = inner(residual, delta, step, cache, **kw)
+            seen.append(residual.clone().cpu())
+            return out
+        block.forward = wrapped
+    from ginfer_amd import StepEntry
+    runner.step([StepEntry("a", ids, [0])])
+    want = pp.residual_streams(ids, pp.read_weights(folders[name]), pp.read_config(folders[name]))
+    assert len(seen) == want.shape[0] == 5
+    for i, s in enumerate(seen):
+        assert H.rel_err(s, want[i]) < 1e-5, "after layer %d" % i
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["mix", "wide", "deep"])
+def test_unequal_requests_together_with_pages_and_slots_used_again(folders, name, dtype):
+    """Seven requests through three state slots and a pool that holds three of them: portions of some beside single
+    tokens of others, requests that sit a step out, and every page and slot used several times."""
+    reqs = requests_for(name, [70, 3, 120, 33, 64, 17, 90], seed=50)
+    steps = H.steps_mixed(reqs, max_live=3, seed=4)
+    ps = CONFIGS[name][1]
+    tokens = H.max_live_tokens(steps, round_to=ps)
+    runner = runner_for(folders[name], name, dtype, tokens=tokens, max_requests=3)
+    alone = H.run_steps(runner_for(folders[name], name, dtype), H.steps_whole(reqs)) if dtype == "float32" else None
+    for rounds in range(2):                      # the second time the steps' shapes are known and recorded
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        compare(got, reqs, folders[name], TOL[dtype], "%s %s mixed, round %d" % (name, dtype, rounds), CLOSE[dtype])
+        if alone is not None:
+            for key, row in alone.items():
+                assert np.array_equal(row, got[key]), "%s: in a batch, %s differs from the request alone" % (name, key)
+    assert not runner.cache.requests
+
+
+def drawn_config(seed):
+    """A configuration drawn at random."""
+    rng = np.random.RandomState(seed)
+    pick = lambda *xs: xs[rng.randint(len(xs))]
+    width = int(pick(24, 40, 50, 52, 64, 66, 96, 136, 75))
+    layers = []
+    for _ in range(int(rng.randint(1, 6))):
+        ff = pick(None, 16, 36, 37, 64, 100)
+        kind = pick("gla", "retention", "attention")
+        heads = int(pick(1, 2, 3, 4, 6))
+        dim, vdim = int(pick(2, 4, 7, 8, 12, 16, 32, 56, 72)), int(pick(1, 4, 5, 8, 20, 32, 48, 80))
+        dims = int(pick(2, 4, dim - dim % 2)) if dim >= 4 else 2
+        rot = pick(None, (float(pick(10.0, 1e3, 2.5e5)), min(dims, dim - dim % 2)))
+        if kind == "gla":
+            layers.append((GLA(heads, dim, vdim, float(pick(1.0, 3.0, 16.0)), rank=int(pick(1, 2, 5, 16))), ff))
+        elif kind == "retention":
+            layers.append((RET(heads, dim, vdim, [float(1 - 2.0 ** -rng.randint(1, 9)) for _ in range(heads)], rot=rot), ff))
+        else:
+            kv = int(pick(*[d for d in (1, 2, 3, 4, 6) if heads % d == 0]))
+            layers.append((ATT(heads, kv, dim, vdim, float(pick(0.1, 0.25, 0.5)), int(pick(1, 2, 7, 16, 40, 100)),
+                               int(pick(1, 2, 5, 8, 12, 50)), rot=rot), ff))
+    return config(width, int(pick(50, 128, 301)), layers, eps=float(pick(1e-6, 1e-5, 1e-4)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(12))
+def test_configurations_drawn_at_random(tmp_path, seed, dtype):
+    cfg = drawn_config(seed)
+    folder = make_folder(tmp_path / "m", cfg, seed=seed)
+    reqs = {"q%d" % i: H.random_tokens(n, cfg["vocab"], 200 + seed + i) for i, n in enumerate([1, 23, 70])}
+    from ginfer_amd import ModelRunner
+    page = [8, 16, 32][seed % 3]
+    runner = ModelRunner(folder, dtype=dtype, page_size=page, num_pages=-(-256 // page), max_requests=3, max_model_len=512)
+    for what, steps in (("whole", H.steps_whole(reqs)), ("decoded", H.steps_last_decoded(reqs, last=20)),
+                        ("mixed", H.steps_mixed(reqs, max_live=3, seed=seed))):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        compare(got, reqs, folder, TOL[dtype], "drawn configuration %d (%s) %s %s" % (seed, json.dumps(cfg), dtype, what),
+                2 * CLOSE[dtype], median=1.0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """A short prompt and 400 decoded tokens, recorded steps replayed throughout: windows pass over decoded tokens, blocks
+    fill and are seen, pages behind the window go back."""
+    reqs = requests_for("mix", [420], seed=70)
+    runner = runner_for(folders["mix"], "mix", dtype)
+    got = H.run_steps(runner, H.steps_last_decoded(reqs, last=400))
+    compare(got, reqs, folders["mix"], TOL[dtype], "long decoding " + dtype, CLOSE[dtype])
+    if runner.use_graphs:
+        assert runner.counts["replayed_decode"] > 300
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_far_block_decides_the_last_token(tmp_path, dtype):
+    """One attention layer whose keys are the tokens themselves: the last token's query matches the key of one marked
+    token, which sits in a block hundreds of tokens back, at a page's edge, among the first tokens, just behind the window
+    in a block that is seen, or in a block that is not seen yet (then nothing of it may show); whole and decoded."""
+    size, pool = 24, 5
+    cfg = config(32, 40, [(ATT(2, 1, 16, 16, 4.0, size, pool), None)])
+    T = 260
+    lo = T - size                                     # 236: blocks 0..46 end before it (47 * 5 = 235); 235 is unseen
+    for place, seen in ((0, True), (63, True), (64, True), (200, True), (234, True), (235, False), (236, True)):
+        def edit(t, place=place):
+            for n in t:
+                if n.endswith("norm1") or n == "final.norm":
+                    t[n].zero_()
+            e = t["embed"]
+            e.copy_((torch.randn(e.shape, generator=torch.Generator().manual_seed(1)) * 0.2).to(e.dtype))
+            e[:, :2] = 0
+            e[7].zero_()
+            e[8].zero_()
+            e[7, 1] = 4.0                              # token 7: the marked key (keys read coordinate 1)
+            e[8, 0] = 4.0                              # token 8, the last: the query that matches it (queries read coordinate 0)
+            for n in ("q", "k"):
+                t["l0.mix." + n].zero_()
+            t["l0.mix.q"][0::16, 0] = 1.0              # coordinate 0 of each head's query
+            t["l0.mix.k"][0, 1] = 1.0
+            t["l0.mix.pb"].fill_(-12.0)
+            t["l0.mix.g"].zero_()
+            t["l0.rg1"].zero_()
+            t["l0.rg1.b"].fill_(4.0)
+            t["l0.mix.v"] *= 30                        # what the marked token brings is as large as the stream itself
+            t["l0.mix.o"] *= 30
+        folder = make_folder(tmp_path / ("m%d" % place), cfg, seed=3, std_scale=1.0, edit=edit)
+        ids = [int(x) % 6 for x in H.random_tokens(T, 40, place)]
+        ids[place] = 7
+        ids[-1] = 8
+        reqs = {"a": ids}
+        runner = runner_for(folder, "wide", dtype, tokens=512)
+        for what, steps in (("whole", H.steps_whole(reqs)), ("decoded", H.steps_last_decoded(reqs, last=30))):
+            got = H.run_steps(runner, steps)
+            compare(got, reqs, folder, TOL[dtype], "marked token at %d, %s, %s" % (place, what, dtype))
+        moved = list(ids)
+        moved[place] = 1
+        changed = H.rel_err(plain(folder, moved)[-1], plain(folder, ids)[-1])
+        assert (changed > 0.02) == seen, (place, changed)       # the plain statement sees the token, or rightly not
+
+
+LARGER = config(384, 1000, [
+    (GLA(6, 64, 128, 16.0, rank=16), 512),
+    (ATT(12, 4, 128, 64, 0.12, 300, 32, rot=(250000.0, 64)), 640),
+    (RET(3, 128, 80, (0.98, 0.995, 0.999), rot=(1e4, 32)), None),
+    (ATT(6, 6, 48, 80, 0.2, 1000, 100, rot=(500.0, 16)), 512),
+], eps=1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_at_larger_sizes(tmp_path, dtype):
+    """1,300 tokens at once (products of many rows, many windows and blocks), then 30 decoded tokens and a second request
+    in portions beside them."""
+    folder = make_folder(tmp_path / "m", LARGER, seed=11, std_scale=2.0, edit=lambda t: sharpen(t, 2.0))
+    reqs = {"long": H.random_tokens(1330, 1000, 1), "short": H.random_tokens(150, 1000, 2)}
+    from ginfer_amd import ModelRunner, StepEntry
+    runner = ModelRunner(folder, dtype=dtype, page_size=16, num_pages=-(-1600 // 16), max_requests=4, max_model_len=1600)
+    got = {}
+    logits = runner.step([StepEntry("long", reqs["long"][:1300], [0, 1, 640, 1299])]).cpu().numpy()
+    got.update({("long", p): row for p, row in zip([0, 1, 640, 1299], logits)})
+    at = 0
+    for k in range(30):
+        n = min(7, 150 - at)
+        entries = [StepEntry("long", reqs["long"][1300 + k:1301 + k], [0])] + ([StepEntry("short", reqs["short"][at:at + n], [n - 1])] if n else [])
+        logits = runner.step(entries).cpu().numpy()
+        got[("long", 1300 + k)] = logits[0]
+        if n:
+            got[("short", at + n - 1)] = logits[1]
+            at += n
+    runner.cache.check()
+    worst = []
+    for (rid, p), row in sorted(got.items()):
+        ref = plain(folder, reqs[rid])
+        worst.append(float(np.abs(row.astype(np.float64) - ref[p]).max() / np.abs(ref).max()))
+    assert np.isfinite(worst).all()
+    if dtype == "float32":
+        assert max(worst) < TOL[dtype], worst
+    else:
+        assert float(np.median(worst)) < TOL[dtype] / 2 and sum(w > TOL[dtype] for w in worst) <= 0.1 * len(worst), worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_steps_equal_launched_ones(folders, dtype):
+    reqs = requests_for("mix", [60, 25, 41], seed=80)
+    steps = H.steps_mixed(reqs, max_live=3, seed=9)
+    outs = []
+    for graphs in (True, False):
+        runner = runner_for(folders["mix"], "mix", dtype, use_graphs=graphs)
+        for rounds in range(3):
+            got = H.run_steps(runner, steps)
+        outs.append(got)
+        if graphs:
+            assert runner.use_graphs and runner.counts["replayed_decode"] + runner.counts["replayed_padded"] > 0
+    for key, row in outs[0].items():
+        if dtype == "float32":
+            assert np.array_equal(row, outs[1][key]), key
+    if dtype == "bfloat16":
+        compare(outs[0], reqs, folders["mix"], TOL[dtype], "recorded", CLOSE[dtype])
+        compare(outs[1], reqs, folders["mix"], TOL[dtype], "launched", CLOSE[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_program(folders, tmp_path, dtype):
+    reqs = requests_for("mix", [40, 9, 77], seed=90)
+    steps = H.steps_mixed(reqs, max_live=2, seed=2)
+    cfg_vocab = CONFIGS["mix"][0]["vocab"]
+    import plain_model
+    orig = plain_model.read_config
+    plain_model.read_config = lambda folder: {"vocab_size": cfg_vocab}          # the helper only asks for the vocabulary
+    try:
+        got = H.run_trace(folders["mix"], dtype, steps, tmp_path / "out", H.max_live_tokens(steps), page_size=16)
+    finally:
+        plain_model.read_config = orig
+    compare(got, reqs, folders["mix"], TOL[dtype], "trace replay " + dtype, CLOSE[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(folders, dtype):
+    """Engine.generate with its scheduler: five prompts through three slots under a budget of 48 tokens a step.  Every
+    token is the plain statement's greedy choice after the engine's own tokens so far (in bfloat16: or within rounding
+    of it)."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    name = "mix"
+    folder = folders[name]
+    prompts = list(requests_for(name, [3, 30, 11, 64, 1], seed=100).values())
+    eng = Engine(EngineConfig(model_path=folder, dtype=dtype, max_num_batched_tokens=48, max_num_seqs=3, max_seq_len=256,
+                              kvcache_block_size=8, num_kvcache_blocks=96))
+    outs = eng.generate(prompts, SamplingParams(max_tokens=24, ignore_eos=True))
+    cfg, w = pp.read_config(folder), pp.read_weights(folder)
+    far = 0
+    for p, o in zip(prompts, outs):
+        assert len(o.token_ids) == 24
+        logits = pp.logits((p + o.token_ids)[:-1], w, cfg)
+        for k, tok in enumerate(o.token_ids):
+            row = logits[len(p) - 1 + k]
+            best = int(torch.argmax(row))
+            gap = float(row[best] - row[tok]) / float(row.abs().max())
+            if dtype == "float32":
+                assert tok == best or gap <= 1e-5, "token %d after a prompt of %d: engine %d, plain %d (gap %.3g)" % (k, len(p), tok, best, gap)
+            else:
+                far += not (tok == best or gap <= 6e-2)
+    assert far <= 3
+    eng.runner.cache.check()
+
+
+def test_command_line_generates(folders):
+    import subprocess
+    import sys
+    folder = folders["deep"]
+    cmd = [sys.executable, os.path.join(H.ROOT, "bin", "ginfer"), "generate", "--model-path", folder, "--dtype", "float32",
+           "--prompt-ids", "1,2,3,4,5", "--max-tokens", "6", "--ignore-eos", "--max-num-seqs", "2", "--max-seq-len", "64",
+           "--num-kvcache-blocks", "16"]
+    out = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    cfg, w = pp.read_config(folder), pp.read_weights(folder)
+    ids = [1, 2, 3, 4, 5]
+    for _ in range(6):
+        ids.append(int(torch.argmax(pp.logits(ids, w, cfg)[-1])))
+    assert json.loads(out.stdout.strip().splitlines()[0])["token_ids"] == ids[5:]
