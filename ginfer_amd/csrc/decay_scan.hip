@@ -111,21 +111,43 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
   }
 }
 
-// decay[t, c] = exp(-softplus(-z) / tau), z = sum_r a2[c, r] * low[t, r] + bias[c]
+// decay[t, c] = exp(-softplus(-z) / tau), z = sum_r a2[c, r] * low[t, r] + bias[c].  A workgroup takes GD_TOKENS tokens and 256
+// channels: a thread keeps its channel's row of a2 in registers (ranks up to GD_RANK; longer rows are read again per token)
+// and the tokens' narrow rows go through LDS, so a2 comes from memory once per GD_TOKENS tokens.
+#define GD_TOKENS 16
+#define GD_RANK 64
 __global__ __launch_bounds__(256) void gla_decay_kernel(float* __restrict__ decay, const float* __restrict__ low,
                                                         int64_t low_stride, const float* __restrict__ a2,
-                                                        const float* __restrict__ bias, int channels, int rank,
+                                                        const float* __restrict__ bias, int tokens, int channels, int rank,
                                                         float inv_tau) {
-  const int64_t t = blockIdx.x;
-  const float* lo = low + t * low_stride;
-  for (int c = threadIdx.x; c < channels; c += 256) {
-    const float* w = a2 + (int64_t)c * rank;
+  extern __shared__ float lows[];                      // [GD_TOKENS][rank]
+  const int t0 = blockIdx.x * GD_TOKENS, nt = min(GD_TOKENS, tokens - t0);
+  for (int idx = threadIdx.x; idx < nt * rank; idx += 256) lows[idx] = low[(int64_t)(t0 + idx / rank) * low_stride + idx % rank];
+  __syncthreads();
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= channels) return;
+  const float* w = a2 + (int64_t)c * rank;
+  float wr[GD_RANK];
+  const bool kept = rank <= GD_RANK;
+  if (kept) {
+#pragma unroll
+    for (int r = 0; r < GD_RANK; ++r) wr[r] = r < rank ? w[r] : 0.f;
+  }
+  const float b = bias[c];
+  for (int tt = 0; tt < nt; ++tt) {
+    const float* lo = lows + tt * rank;
     float z = 0.f;
-    for (int r = 0; r < rank; ++r) z = fmaf(w[r], lo[r], z);
-    z += bias[c];
+    if (kept) {
+#pragma unroll
+      for (int r = 0; r < GD_RANK; ++r)
+        if (r < rank) z = fmaf(wr[r], lo[r], z);
+    } else {
+      for (int r = 0; r < rank; ++r) z = fmaf(w[r], lo[r], z);
+    }
+    z += b;
     // log(sigmoid(z)) = -softplus(-z); far out the softplus is its argument
     const float sp = -z > 30.f ? -z : log1pf(expf(-z));
-    decay[t * channels + c] = expf(-sp * inv_tau);
+    decay[(int64_t)(t0 + tt) * channels + c] = expf(-sp * inv_tau);
   }
 }
 
@@ -188,8 +210,10 @@ extern "C" int ga_gla_decay(void* decay, const void* low, int64_t low_stride, co
                             int channels, int rank, float tau, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (channels <= 0 || rank <= 0 || !(tau > 0.f)) return -1;
-  hipLaunchKernelGGL(gla_decay_kernel, dim3(tokens), dim3(256), 0, stream, (float*)decay, (const float*)low, low_stride,
-                     (const float*)a2, (const float*)bias, channels, rank, 1.0f / tau);
+  if ((size_t)GD_TOKENS * rank * sizeof(float) > 48 * 1024) return -2;
+  dim3 grid((tokens + GD_TOKENS - 1) / GD_TOKENS, (channels + 255) / 256);
+  hipLaunchKernelGGL(gla_decay_kernel, grid, dim3(256), GD_TOKENS * rank * sizeof(float), stream, (float*)decay,
+                     (const float*)low, low_stride, (const float*)a2, (const float*)bias, tokens, channels, rank, 1.0f / tau);
   return GA_CHECK_LAUNCH();
 }
 

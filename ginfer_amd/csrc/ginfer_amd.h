@@ -247,10 +247,11 @@ int ga_head_norm_gate(void* out, const void* x, const void* weight, const void* 
 
 // ---- pooled_attention.hip: attention over a window of tokens and the means of the blocks before it, sigmoid weights.
 // prepare: q and k of a 32-bit projection [q heads | k heads | v heads ...] turned by position (pairs 2i, 2i + 1), divided by
-// their root mean square per head where `unit`; q out float [tokens, nh dim]; k, v into rows [slot][nkv][dim | vdim]
+// their root mean square per head where `unit`; q out float [tokens, nh dim]; k into rows [slot][nkv][dim], v transposed inside
+// its page [page][nkv][vdim][slot]
 int ga_pwa_prepare(void* q_out, const void* proj, int64_t stride, const void* positions, const void* cos_t, const void* sin_t,
                    const void* slot_mapping, void* k_rows, void* v_rows, int tokens, int nh, int nkv, int dim, int vdim,
-                   int rot_dims, int unit, float eps, int write, int cache_bf16, hipStream_t stream);
+                   int rot_dims, int unit, float eps, int write, int page_size, int cache_bf16, hipStream_t stream);
 // for every token that ends a block of `pool` positions: the block's mean key and value (float rows at pool_slots[token])
 int ga_pwa_pool(void* pk_rows, void* pv_rows, const void* k_rows, const void* v_rows, const void* positions,
                 const void* token_entry, const void* table, int width, const void* pool_slots, int tokens, int nkv, int dim,
@@ -261,6 +262,15 @@ int ga_pwa_attend(void* out, const void* q, const void* k_rows, const void* v_ro
                   int pool_width, const void* head_bias, const void* gate, int64_t gate_stride, int tokens, int nh, int nkv,
                   int dim, int vdim, int size, int pool, int page_size, float scale, int cache_bf16, int out_bf16,
                   hipStream_t stream);
+
+// the same on the matrix cores (bfloat16 cache and output): prompt portions by the step's tiles int32 [n_tiles][4] = (entry,
+// first row, rows, first position), single tokens by info int32 [n_single][4] = (row, position, entry, -), their keys dealt to
+// `splits` workgroups (partial: float [splits][n_single][nh vdim] where splits > 1); dim a multiple of 8, page_size too
+int ga_pwa_attend_mfma(void* out, void* partial, const void* q, const void* k_rows, const void* v_pages, const void* pk_rows,
+                       const void* pv_pages, const void* tiles, int n_tiles, const void* info, int n_single, int splits,
+                       const void* table, int width, const void* pool_table, int pool_width, const void* head_bias,
+                       const void* gate, int64_t gate_stride, int nh, int nkv, int dim, int vdim, int size, int pool,
+                       int page_size, float scale, hipStream_t stream);
 
 // ---- gated_residual.hip: residual float [tokens, hidden] += sigmoid(z[:, :hidden]) * y1 (+ sigmoid(z[:, hidden:]) * y2, y2
 // may be null); with next: next = rmsnorm(residual) * next_gain (float [hidden])

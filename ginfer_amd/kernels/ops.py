@@ -1337,11 +1337,12 @@ def _token_rows(t, width, name, dtype=None):
 
 
 def pooled_attention_prepare(proj, positions, cos, sin, slot_mapping, k_rows, v_rows, num_heads, num_kv_heads, dim, vdim, eps,
-                             unit_norm=True, write=True):
+                             page_size, unit_norm=True, write=True):
     """Behind a float32 projection whose first columns are [q heads | k heads | v heads]: q and k turned by position on their
     first r coordinates (pairs 2i, 2i + 1; cos, sin float32 [positions, r / 2], None: no rotation), then divided by their
-    root mean square per head (unit_norm); k and v are written into their rows ([slot][kv head][dim | vdim], float32 or
-    bfloat16) at slot_mapping.  Returns q float32 [T, num_heads * dim]."""
+    root mean square per head (unit_norm); k and v are written into their pages (keys [page][slot][kv head][dim], values
+    transposed inside a page [page][kv head][vdim][slot]; float32 or bfloat16) at slot_mapping.  Returns q float32 [T,
+    num_heads * dim]."""
     _dev(proj, positions, cos, sin, slot_mapping, k_rows, v_rows)
     T = proj.shape[0]
     _rows_of(proj, 0, (num_heads + num_kv_heads) * dim + num_kv_heads * vdim, "q | k | v")
@@ -1366,8 +1367,16 @@ def pooled_attention_prepare(proj, positions, cos, sin, slot_mapping, k_rows, v_
     lib = build.load("pooled_attention")
     _check(lib.ga_pwa_prepare(_ptr(q), _ptr(proj), _i64(proj.stride(0)), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
                               _ptr(k_rows), _ptr(v_rows), _i(T), _i(num_heads), _i(num_kv_heads), _i(dim), _i(vdim), _i(rot),
-                              _i(1 if unit_norm else 0), _f(eps), _i(1 if write else 0), _i(cache_bf16), _stream()), "pwa_prepare")
+                              _i(1 if unit_norm else 0), _f(eps), _i(1 if write else 0), _i(page_size), _i(cache_bf16), _stream()),
+           "pwa_prepare")
     return q
+
+
+def pooled_attention_mfma_supported(dtype, cache_dtype, num_heads, num_kv_heads, dim, page_size):
+    """Whether the matrix-core kernels take these sizes: bfloat16, at most 16 heads to a kv head, keys whose width is a
+    multiple of 8 (a lane's 16 bytes), pages of a multiple of 8 tokens (8 consecutive tokens of a value column lie in one)."""
+    return (dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and num_heads // num_kv_heads <= 16 and dim % 8 == 0
+            and page_size % 8 == 0)
 
 
 def _table(t, entries, name):
@@ -1427,6 +1436,25 @@ def pooled_attention(q, k_rows, v_rows, pk_rows, pv_rows, step, table, pool_tabl
     _need(size >= 1 and pool >= 1 and page_size >= 1, "size, pool and page_size must be positive")
     out = torch.empty((T, num_heads * vdim), dtype=dtype, device=q.device)
     lib = build.load("pooled_attention")
+    if pooled_attention_mfma_supported(dtype, k_rows.dtype, num_heads, num_kv_heads, dim, page_size):
+        # the matrix cores: prompt portions by the step's tiles of 16 rows, single tokens with a kv group's heads side by side
+        plan = _attention_plan(step, PLAN_TILE_ROWS, q.device)
+        n_tiles, n_single = plan["n_tiles"], plan["n_decode"]
+        splits, partial = 1, None
+        if n_single:
+            # the longest walk in tiles of 32: the window and the blocks of the longest context of the step's bucket
+            span = int(plan.get("decode_span") or step.max_kv_len)
+            tiles = (min(size, span) + 31) // 32 + 1 + (span // pool + 31) // 32
+            splits = max(1, min(tiles // TUNING.pooled_decode_tiles_per_split,
+                                TUNING.pooled_decode_workgroups // max(n_single * num_kv_heads, 1), 64))
+            if splits > 1:
+                partial = torch.empty((splits, n_single, num_heads * vdim), dtype=torch.float32, device=q.device)
+        _check(lib.ga_pwa_attend_mfma(_ptr(out), _ptr(partial), _ptr(q), _ptr(k_rows), _ptr(v_rows), _ptr(pk_rows), _ptr(pv_rows),
+                                      _ptr(plan["tiles"]), _i(n_tiles), _ptr(plan["decode_info"]), _i(n_single), _i(splits),
+                                      _ptr(table), _i(width), _ptr(pool_table), _i(pool_width), _ptr(head_bias), _ptr(gate),
+                                      _i64(proj.stride(0) if proj is not None else 0), _i(num_heads), _i(num_kv_heads), _i(dim),
+                                      _i(vdim), _i(size), _i(pool), _i(page_size), _f(scale), _stream()), "pwa_attend_mfma")
+        return out
     _check(lib.ga_pwa_attend(_ptr(out), _ptr(q), _ptr(k_rows), _ptr(v_rows), _ptr(pk_rows), _ptr(pv_rows), _ptr(step.positions),
                              _ptr(step.token_entry), _ptr(table), _i(width), _ptr(pool_table), _i(pool_width), _ptr(head_bias),
                              _ptr(gate), _i64(proj.stride(0) if proj is not None else 0), _i(T), _i(num_heads), _i(num_kv_heads),

@@ -120,6 +120,11 @@ class Tuning:
     # workgroup of it streams from memory no faster than any other), at most `latent_decode_max_splits` to a token
     latent_decode_workgroups: int = 1024
     latent_decode_max_splits: int = 32
+    # attention over a window and pooled blocks, single tokens on the matrix cores: a workgroup is one wavefront that holds a
+    # kv group's heads of one token; the token's tiles of 32 keys are dealt to as many workgroups as bring the launch to about
+    # `pooled_decode_workgroups`, each with at least `pooled_decode_tiles_per_split` tiles (the partial sums just add)
+    pooled_decode_workgroups: int = 2048
+    pooled_decode_tiles_per_split: int = 4
     # ---- routed feed-forwards (parts/mlp.py).  Steps of fewer rows than this run every expert over every row in one
     # product (rows that an expert does not own enter with zeros): no step that is recorded is longer, and up to some
     # hundred rows the experts' weights, which all come from memory either way, are what the step waits for.  Longer steps

@@ -75,7 +75,7 @@ class PooledWindowAttention(Part):
         proj = linear(x, self.w_in, None, out_dtype=torch.float32)
         cos, sin = self.position.tables() if self.position is not None else (None, None)
         q = ops.pooled_attention_prepare(proj, step.positions, cos, sin, near.slot_mapping, k_rows, v_rows, self.nh, self.nkv,
-                                         self.hd, self.vd, self.eps, unit_norm=self.unit_norm, write=near.owner)
+                                         self.hd, self.vd, self.eps, near.page_size, unit_norm=self.unit_norm, write=near.owner)
         if means.owner:
             ops.pooled_attention_pool(pk_rows, pv_rows, k_rows, v_rows, step, near.block_table, means.slot_mapping, self.nkv,
                                       self.hd, self.vd, self.pool, near.page_size)

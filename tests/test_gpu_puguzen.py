@@ -307,7 +307,7 @@ class _AttentionCase:
             rows = range(at, at + n)
             p = proj[at:at + n].cuda()
             q = ops.pooled_attention_prepare(p, step.positions, cos, sin, self.slots(self.table, rows), self.k_rows, self.v_rows,
-                                             self.nh, self.nkv, self.dim, self.vdim, eps, unit_norm=unit)
+                                             self.nh, self.nkv, self.dim, self.vdim, eps, self.page, unit_norm=unit)
             ops.pooled_attention_pool(self.pk, self.pv, self.k_rows, self.v_rows, step, self.table,
                                       self.slots(self.pool_table, [r // self.pool for r in rows]), self.nkv, self.dim, self.vdim,
                                       self.pool, self.page)
@@ -351,7 +351,8 @@ def test_attention_over_window_and_blocks_whole_and_cut(nh, nkv, dim, vdim, size
         case = _AttentionCase(nh, nkv, dim, vdim, size, pool, page, dt, T)
         outs.append(case.run(proj, cuts, bias.cuda(), 0.3, gate_start=gate0))
         assert H.rel_err(outs[-1], want.reshape(T, -1)) < tol, cuts[:4]
-    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    if dtype == "float32":      # bfloat16: portions and single tokens go to different kernels of the matrix cores
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -414,12 +415,13 @@ def test_rotation_of_neighbours_and_unit_norm_before_the_cache():
             v_rows = torch.zeros((40, nkv * vdim), dtype=dt, device="cuda")
             slots = torch.tensor([31, 2, 5, 39, 0, -1, 7, 8, 9], dtype=torch.int64, device="cuda")
             positions = torch.arange(first, first + T, dtype=torch.int32, device="cuda")
-            got = ops.pooled_attention_prepare(proj.cuda(), positions, cos, sin, slots, k_rows, v_rows, nh, nkv, dim, vdim, 1e-5)
+            got = ops.pooled_attention_prepare(proj.cuda(), positions, cos, sin, slots, k_rows, v_rows, nh, nkv, dim, vdim, 1e-5, 8)
             assert H.rel_err(got.cpu(), q.reshape(T, -1)) < 2e-6
             keep = [i for i, s in enumerate(slots.tolist()) if s >= 0]
             rows = [slots[i].item() for i in keep]
             assert H.rel_err(k_rows[rows].float().cpu(), k.reshape(T, -1)[keep]) < tol
-            assert H.rel_err(v_rows[rows].float().cpu(), v[keep]) < tol
+            v_back = v_rows.view(5, nkv, vdim, 8).permute(0, 3, 1, 2).reshape(40, nkv * vdim)      # pages of 8 rows, values transposed inside
+            assert H.rel_err(v_back[rows].float().cpu(), v[keep]) < tol
             untouched = [r for r in range(40) if r not in rows]
             assert float(k_rows[untouched].abs().max()) == 0.0          # a token without a slot writes nothing
 
