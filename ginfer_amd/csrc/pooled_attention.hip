@@ -110,7 +110,7 @@ __device__ __forceinline__ int64_t pa_row(const int32_t* __restrict__ table, int
 
 // grid (tokens, 2 nkv): the keys' and the values' heads of the block that a token ends
 template <typename TC>
-__global__ __launch_bounds__(PA_THREADS) void pwa_pool_kernel(float* __restrict__ pk_rows, float* __restrict__ pv_rows,
+__global__ __launch_bounds__(256) void pwa_pool_kernel(float* __restrict__ pk_rows, float* __restrict__ pv_rows,
                                                               const TC* __restrict__ k_rows, const TC* __restrict__ v_rows,
                                                               const int32_t* __restrict__ positions,
                                                               const int32_t* __restrict__ token_entry,
@@ -126,7 +126,7 @@ __global__ __launch_bounds__(PA_THREADS) void pwa_pool_kernel(float* __restrict_
   const bool keys = blockIdx.y < (unsigned)nkv;
   const int g = keys ? blockIdx.y : blockIdx.y - nkv, w = keys ? dim : vdim;
   const float inv = 1.0f / (float)pool;
-  for (int c = threadIdx.x; c < w; c += PA_THREADS) {
+  for (int c = threadIdx.x; c < w; c += blockDim.x) {
     float sum = 0.f;
     for (int p = pos + 1 - pool; p <= pos; ++p) {
       const int64_t r = pa_row(table, width, e, p, page_size);
@@ -238,7 +238,8 @@ extern "C" int ga_pwa_pool(void* pk_rows, void* pv_rows, const void* k_rows, con
                            int nkv, int dim, int vdim, int pool, int page_size, int cache_bf16, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (nkv <= 0 || 2 * nkv > 65535 || dim <= 0 || vdim <= 0 || pool <= 0 || page_size <= 0 || width <= 0) return -1;
-  dim3 grid(tokens, 2 * nkv), block(PA_THREADS);
+  const int widest = dim > vdim ? dim : vdim;          // a thread a channel: the chains of a block's sum run side by side
+  dim3 grid(tokens, 2 * nkv), block(widest <= 64 ? 64 : widest <= 128 ? 128 : 256);
 #define GO(T) hipLaunchKernelGGL(pwa_pool_kernel<T>, grid, block, 0, stream, (float*)pk_rows, (float*)pv_rows,            \
                                  (const T*)k_rows, (const T*)v_rows, (const int32_t*)positions, (const int32_t*)token_entry, \
                                  (const int32_t*)table, width, (const int64_t*)pool_slots, nkv, dim, vdim, pool, page_size)
@@ -469,12 +470,12 @@ __global__ __launch_bounds__(WAVE) void pwa_heads_kernel(bf16_t* __restrict__ ou
     }
 }
 
-// out[row, h, :] = gate * (partial[0] + partial[1] + ...): a workgroup a record
+// out[row, h, :] = gate * (partial[0] + partial[1] + ...): grid (records, pieces of a row)
 __global__ __launch_bounds__(256) void pwa_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial,
                                                         const int32_t* __restrict__ info, const float* __restrict__ gate,
                                                         int64_t gate_stride, int records, int splits, int width) {
   const int64_t d = blockIdx.x, row = info[4 * d];
-  for (int x = threadIdx.x; x < width; x += 256) {
+  for (int x = blockIdx.y * 256 + threadIdx.x; x < width; x += 256 * gridDim.y) {
     float a = 0.f;
     for (int s = 0; s < splits; ++s) a += partial[((int64_t)s * records + d) * width + x];
     if (gate) a *= pa_sigmoid(gate[row * gate_stride + x]);
@@ -509,7 +510,7 @@ extern "C" int ga_pwa_attend_mfma(void* out, void* partial, const void* q, const
 #undef TAIL
 #undef ARGS
   if (n_single > 0 && splits > 1)
-    hipLaunchKernelGGL(pwa_merge_kernel, dim3(n_single), dim3(256), 0, stream, (bf16_t*)out, (const float*)partial,
+    hipLaunchKernelGGL(pwa_merge_kernel, dim3(n_single, (nh * vdim + 255) / 256 > 64 ? 64 : (nh * vdim + 255) / 256), dim3(256), 0, stream, (bf16_t*)out, (const float*)partial,
                        (const int32_t*)info, (const float*)gate, gate_stride, n_single, splits, nh * vdim);
   return GA_CHECK_LAUNCH();
 }
