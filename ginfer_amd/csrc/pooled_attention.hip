@@ -128,10 +128,18 @@ __global__ __launch_bounds__(256) void pwa_pool_kernel(float* __restrict__ pk_ro
   const float inv = 1.0f / (float)pool;
   for (int c = threadIdx.x; c < w; c += blockDim.x) {
     float sum = 0.f;
-    for (int p = pos + 1 - pool; p <= pos; ++p) {
-      const int64_t r = pa_row(table, width, e, p, page_size);
-      if (r >= 0) sum += keys ? Num<TC>::ld(k_rows + (r * nkv + g) * (int64_t)w + c)
-                              : Num<TC>::ld(v_rows + pa_value_at(r, g, c, nkv, vdim, page_size));
+    // eight rows are asked for at a time and added in the order of the positions
+    for (int p0 = pos + 1 - pool; p0 <= pos; p0 += 8) {
+      float x[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int64_t r = p0 + j <= pos ? pa_row(table, width, e, p0 + j, page_size) : -1;
+        x[j] = r < 0 ? 0.f : keys ? Num<TC>::ld(k_rows + (r * nkv + g) * (int64_t)w + c)
+                                  : Num<TC>::ld(v_rows + pa_value_at(r, g, c, nkv, vdim, page_size));
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (p0 + j <= pos) sum += x[j];
     }
     if (keys) pk_rows[(dst_row * nkv + g) * (int64_t)w + c] = sum * inv;
     else pv_rows[pa_value_at(dst_row, g, c, nkv, vdim, page_size)] = sum * inv;
