@@ -10,7 +10,7 @@
 // through LDS, every thread keeps the state of one column and every 16th row in registers, and the rows' partial
 // outputs are added in a fixed order.  So a token's result does not depend on how the request's tokens were cut into
 // steps, nor on what else is in the batch.
-// gla_decay: a = sigmoid(z)^(1/tau), z = A2 (low) + b, `low` being the rows of a narrow projection (32-bit), as
+// gla_decay: a = sigmoid(z)^(1/tau), z = A2 (low) + b (A2 handed over transposed), `low` being the rows of a narrow projection (32-bit), as
 //   exp(-softplus(-z) / tau), all in 32-bit.
 // head_norm_gate: out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) (* weight[:]) (* silu(gate[t, h, :])).
 #include "common.h"
@@ -111,43 +111,41 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
   }
 }
 
-// decay[t, c] = exp(-softplus(-z) / tau), z = sum_r a2[c, r] * low[t, r] + bias[c].  A workgroup takes GD_TOKENS tokens and 256
-// channels: a thread keeps its channel's row of a2 in registers (ranks up to GD_RANK; longer rows are read again per token)
-// and the tokens' narrow rows go through LDS, so a2 comes from memory once per GD_TOKENS tokens.
+// decay[t, c] = exp(-softplus(-z) / tau), z = sum_r a2t[r, c] * low[t, r] + bias[c], the sum in ascending r.  a2t is the
+// widening matrix TRANSPOSED, [rank][channels]: neighbouring threads read neighbouring channels.  A workgroup takes GD_TOKENS
+// tokens and 256 channels; the tokens' narrow rows go through LDS and every element of a2t is read once for all of them.
 #define GD_TOKENS 16
-#define GD_RANK 64
 __global__ __launch_bounds__(256) void gla_decay_kernel(float* __restrict__ decay, const float* __restrict__ low,
-                                                        int64_t low_stride, const float* __restrict__ a2,
+                                                        int64_t low_stride, const float* __restrict__ a2t,
                                                         const float* __restrict__ bias, int tokens, int channels, int rank,
                                                         float inv_tau) {
-  extern __shared__ float lows[];                      // [GD_TOKENS][rank]
+  extern __shared__ float lows[];                      // [rank][GD_TOKENS]
   const int t0 = blockIdx.x * GD_TOKENS, nt = min(GD_TOKENS, tokens - t0);
-  for (int idx = threadIdx.x; idx < nt * rank; idx += 256) lows[idx] = low[(int64_t)(t0 + idx / rank) * low_stride + idx % rank];
+  for (int idx = threadIdx.x; idx < GD_TOKENS * rank; idx += 256) {
+    const int tt = idx / rank, r = idx % rank;
+    lows[r * GD_TOKENS + tt] = tt < nt ? low[(int64_t)(t0 + tt) * low_stride + r] : 0.f;
+  }
   __syncthreads();
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= channels) return;
-  const float* w = a2 + (int64_t)c * rank;
-  float wr[GD_RANK];
-  const bool kept = rank <= GD_RANK;
-  if (kept) {
+  float z[GD_TOKENS];
 #pragma unroll
-    for (int r = 0; r < GD_RANK; ++r) wr[r] = r < rank ? w[r] : 0.f;
+  for (int tt = 0; tt < GD_TOKENS; ++tt) z[tt] = 0.f;
+  for (int r = 0; r < rank; ++r) {
+    const float w = a2t[(int64_t)r * channels + c];
+    const float* lo = lows + r * GD_TOKENS;
+#pragma unroll
+    for (int tt = 0; tt < GD_TOKENS; ++tt) z[tt] = fmaf(w, lo[tt], z[tt]);
   }
   const float b = bias[c];
-  for (int tt = 0; tt < nt; ++tt) {
-    const float* lo = lows + tt * rank;
-    float z = 0.f;
-    if (kept) {
 #pragma unroll
-      for (int r = 0; r < GD_RANK; ++r)
-        if (r < rank) z = fmaf(wr[r], lo[r], z);
-    } else {
-      for (int r = 0; r < rank; ++r) z = fmaf(w[r], lo[r], z);
+  for (int tt = 0; tt < GD_TOKENS; ++tt) {
+    if (tt < nt) {
+      const float v = z[tt] + b;
+      // log(sigmoid(v)) = -softplus(-v); far out the softplus is its argument
+      const float sp = -v > 30.f ? -v : log1pf(expf(-v));
+      decay[(int64_t)(t0 + tt) * channels + c] = expf(-sp * inv_tau);
     }
-    z += b;
-    // log(sigmoid(z)) = -softplus(-z); far out the softplus is its argument
-    const float sp = -z > 30.f ? -z : log1pf(expf(-z));
-    decay[(int64_t)(t0 + tt) * channels + c] = expf(-sp * inv_tau);
   }
 }
 
@@ -206,14 +204,14 @@ extern "C" int ga_decay_scan(void* out, const void* q, const void* k, const void
   return GA_CHECK_LAUNCH();
 }
 
-extern "C" int ga_gla_decay(void* decay, const void* low, int64_t low_stride, const void* a2, const void* bias, int tokens,
+extern "C" int ga_gla_decay(void* decay, const void* low, int64_t low_stride, const void* a2t, const void* bias, int tokens,
                             int channels, int rank, float tau, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (channels <= 0 || rank <= 0 || !(tau > 0.f)) return -1;
   if ((size_t)GD_TOKENS * rank * sizeof(float) > 48 * 1024) return -2;
   dim3 grid((tokens + GD_TOKENS - 1) / GD_TOKENS, (channels + 255) / 256);
   hipLaunchKernelGGL(gla_decay_kernel, grid, dim3(256), GD_TOKENS * rank * sizeof(float), stream, (float*)decay,
-                     (const float*)low, low_stride, (const float*)a2, (const float*)bias, tokens, channels, rank, 1.0f / tau);
+                     (const float*)low, low_stride, (const float*)a2t, (const float*)bias, tokens, channels, rank, 1.0f / tau);
   return GA_CHECK_LAUNCH();
 }
 

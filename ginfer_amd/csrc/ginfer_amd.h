@@ -237,9 +237,9 @@ int ga_decay_scan(void* out, const void* q, const void* k, const void* v, int64_
                   const void* head_decay, const void* cos_t, const void* sin_t, int rot_dims, float q_scale, float k_scale,
                   void* state, const void* slots, const void* cu, const void* q_start, int entries, int heads, int dim,
                   int vdim, hipStream_t stream);
-// decay float [tokens, channels] = sigmoid(a2 low + bias)^(1 / tau); low: 32-bit rows of `rank` numbers with a stride; a2
-// float [channels, rank]
-int ga_gla_decay(void* decay, const void* low, int64_t low_stride, const void* a2, const void* bias, int tokens,
+// decay float [tokens, channels] = sigmoid(a2 low + bias)^(1 / tau); low: 32-bit rows of `rank` numbers with a stride; a2t:
+// a2 transposed, float [rank, channels]
+int ga_gla_decay(void* decay, const void* low, int64_t low_stride, const void* a2t, const void* bias, int tokens,
                  int channels, int rank, float tau, hipStream_t stream);
 // out [tokens, heads, vdim] = x / rms(x over vdim) (* weight [vdim], or null) (* silu(gate), 32-bit rows with a stride, or null)
 int ga_head_norm_gate(void* out, const void* x, const void* weight, const void* gate, int64_t gate_stride, int64_t tokens,

@@ -1233,6 +1233,7 @@ def conv_rope_kv(proj, weight, state, slots, step, cos, sin, slot_mapping, k_pag
 
 
 DECAY_SCAN_MAX_DIM = 256
+GLA_DECAY_MAX_RANK = 768       # 16 tokens' narrow rows in 48 KB of LDS
 
 
 def _step_entries(step, slots):
@@ -1251,20 +1252,21 @@ def _rows_of(proj, start, width, name):
     return proj[:, start:start + width]
 
 
-def gla_decay(proj, low_start, a2, bias, tau):
-    """sigmoid(a2 low + bias)^(1 / tau) in 32-bit: low = proj[:, low_start : low_start + rank] (float32 rows), a2 float32
-    [channels, rank], bias float32 [channels].  Returns float32 [T, channels]."""
-    _dev(proj, a2, bias)
-    _need(a2.dim() == 2, "a2 must be [channels, rank]")
-    C, R = a2.shape
-    _f32(a2, (C, R), "a2")
+def gla_decay(proj, low_start, a2t, bias, tau):
+    """sigmoid(a2 low + bias)^(1 / tau) in 32-bit: low = proj[:, low_start : low_start + rank] (float32 rows), a2t the widening
+    matrix transposed, float32 [rank, channels], bias float32 [channels].  Returns float32 [T, channels]."""
+    _dev(proj, a2t, bias)
+    _need(a2t.dim() == 2, "a2t must be [rank, channels]")
+    R, C = a2t.shape
+    _f32(a2t, (R, C), "a2t")
     _f32(bias, (C,), "bias")
+    _need(R <= GLA_DECAY_MAX_RANK, "the decay's narrow projection may be up to %d wide, got %d", GLA_DECAY_MAX_RANK, R)
     low = _rows_of(proj, low_start, R, "low")
     _need(tau > 0, "tau must be positive, got %r", tau)
     T = proj.shape[0]
     out = torch.empty((T, C), dtype=torch.float32, device=proj.device)
     lib = build.load("decay_scan")
-    _check(lib.ga_gla_decay(_ptr(out), _ptr(low), _i64(proj.stride(0)), _ptr(a2), _ptr(bias), _i(T), _i(C), _i(R), _f(tau),
+    _check(lib.ga_gla_decay(_ptr(out), _ptr(low), _i64(proj.stride(0)), _ptr(a2t), _ptr(bias), _i(T), _i(C), _i(R), _f(tau),
                             _stream()), "gla_decay")
     return out
 

@@ -64,8 +64,8 @@ class GatedLinearAttention(_DecayedLinearAttention):
     def __init__(self, hidden_size, num_heads, key_dim, value_dim, decay_rank, tau, eps, dtype, device):
         super().__init__(hidden_size, num_heads, key_dim, value_dim, eps, dtype, device)
         self.rank, self.tau = int(decay_rank), float(tau)
-        if self.rank < 1 or not self.tau > 0:
-            raise ValueError("the decay needs a rank >= 1 and tau > 0, got %r and %r" % (decay_rank, tau))
+        if not 1 <= self.rank <= ops.GLA_DECAY_MAX_RANK or not self.tau > 0:
+            raise ValueError("the decay needs a rank of 1 to %d and tau > 0, got %r and %r" % (ops.GLA_DECAY_MAX_RANK, decay_rank, tau))
         self.w_a2 = self.b_a2 = self.norm_weight = None
 
     def weight_specs(self):
@@ -77,7 +77,7 @@ class GatedLinearAttention(_DecayedLinearAttention):
 
     def bind_weights(self, t):
         self.w_in = torch.cat([t["q"], t["k"], t["v"], t["g"], t["a1"]], dim=0).contiguous()
-        self.w_a2 = t["a2"].float().contiguous()
+        self.w_a2 = t["a2"].float().t().contiguous()        # [rank, channels]: the kernel reads neighbouring channels
         self.b_a2 = t["a2.b"].float().contiguous()
         self.norm_weight = t["norm"].float().contiguous()
         self.w_o = t["o"]

@@ -200,7 +200,7 @@ def test_decay_of_gated_linear_attention():
         proj = torch.randn((tokens, 11 + rank), generator=g)
         a2, b = torch.randn((channels, rank), generator=g) * 3, torch.randn((channels,), generator=g) * 3
         b[0], b[1 % channels] = 60.0, -60.0            # far out on both sides
-        got = ops.gla_decay(proj.cuda(), 11, a2.cuda(), b.cuda(), tau).cpu()
+        got = ops.gla_decay(proj.cuda(), 11, a2.t().contiguous().cuda(), b.cuda(), tau).cpu()
         z = proj[:, 11:].double() @ a2.double().T + b.double()
         want = torch.exp(torch.nn.functional.logsigmoid(z) / tau)
         assert torch.isfinite(got).all() and float((got.double() - want).abs().max()) < 2e-6
