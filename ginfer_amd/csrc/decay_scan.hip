@@ -131,11 +131,18 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(float* __restrict__ deca
   float z[GD_TOKENS];
 #pragma unroll
   for (int tt = 0; tt < GD_TOKENS; ++tt) z[tt] = 0.f;
-  for (int r = 0; r < rank; ++r) {
-    const float w = a2t[(int64_t)r * channels + c];
-    const float* lo = lows + r * GD_TOKENS;
+  for (int r0 = 0; r0 < rank; r0 += 8) {               // eight elements of a2t are asked for at a time
+    float w[8];
 #pragma unroll
-    for (int tt = 0; tt < GD_TOKENS; ++tt) z[tt] = fmaf(w, lo[tt], z[tt]);
+    for (int j = 0; j < 8; ++j) w[j] = r0 + j < rank ? a2t[(int64_t)(r0 + j) * channels + c] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (r0 + j < rank) {
+        const float* lo = lows + (r0 + j) * GD_TOKENS;
+#pragma unroll
+        for (int tt = 0; tt < GD_TOKENS; ++tt) z[tt] = fmaf(w[j], lo[tt], z[tt]);
+      }
+    }
   }
   const float b = bias[c];
 #pragma unroll
