@@ -58,7 +58,7 @@ class Scheduler:
         ps = self.cache.page_size
         grown = min(total, self.max_model_len)
         for gi, g in enumerate(self.cache.groups):
-            need = -(-grown // ps)
+            need = -(-g.rows_for(grown) // ps)      # a group may keep a row per block of positions
             if g.window is not None:         # token by token a window holds the pages that `window` positions can touch
                 need = min(need, self.cache.window_span_pages(g.window, ps))
             if need > g.pool.num_pages:

@@ -756,6 +756,29 @@ def test_greedy_generation_through_the_entry_point(folders, dtype):
     eng.runner.cache.check()
 
 
+def test_pool_planned_from_the_device_memory(folders):
+    """No page counts given: the engine sizes the groups itself (tokens behind a window, rows per block, state slots) and
+    generates what the plain statement generates."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    folder = folders["mix"]
+    eng = Engine(EngineConfig(model_path=folder, dtype="float32", max_num_batched_tokens=64, max_num_seqs=4, max_seq_len=512,
+                              kvcache_block_size=8, gpu_memory_utilization=0.05))
+    groups = {g.spec: g.pool.num_pages for g in eng.runner.cache.groups}
+    assert len(groups) == 4 and all(n >= 1 for n in groups.values())
+    for spec, n in groups.items():
+        if spec.window is not None:
+            assert n == eng.runner.cache.window_pages(spec.window, 8, 4, 64, 512)
+    prompts = list(requests_for("mix", [150, 9], seed=300).values())
+    outs = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    cfg, w = pp.read_config(folder), pp.read_weights(folder)
+    for p, o in zip(prompts, outs):
+        logits = pp.logits((p + o.token_ids)[:-1], w, cfg)
+        for k, tok in enumerate(o.token_ids):
+            row = logits[len(p) - 1 + k]
+            assert tok == int(torch.argmax(row)) or float(row.max() - row[tok]) / float(row.abs().max()) <= 1e-5
+    eng.runner.cache.check()
+
+
 def test_command_line_generates(folders):
     import subprocess
     import sys

@@ -151,6 +151,24 @@ def test_manager_with_rows_that_stand_for_blocks_of_positions():
     assert all(g.pool.num_free == g.pool.num_pages for g in m.groups)
 
 
+def test_pool_planned_for_a_group_of_rows_per_block():
+    """From a number of bytes: the windowed group gets what a window can hold, the group of rows per block of 4 positions a
+    quarter of the pages a group of tokens would get for the same tokens (and one page more per request), at 4 bytes an
+    element whatever the model's format."""
+    near = PagedSpec((("k", 8), ("v", 8)), window=9)
+    means = PagedSpec((("k", 8), ("v", 8)), every=4, dtype=torch.float32)
+    full = PagedSpec((("c", 16),))
+    specs = [StateSpec((2, 2)), [near, means], full]
+    counts = CacheManager.plan_pages(specs, 4, 2, 1 << 20, max_requests=3, max_step_tokens=64, max_model_len=512)
+    by = dict(zip(CacheManager.group_specs(specs), counts))
+    assert by[near] == CacheManager.window_pages(9, 4, 3, 64, 512)
+    assert by[means] == by[full] // 4 + 3 + 1
+    used = by[near] * 16 * 4 * 2 + by[means] * 16 * 4 * 4 + by[full] * 16 * 4 * 2
+    assert 0.9 * (1 << 20) < used <= (1 << 20)
+    m = CacheManager(specs, 4, counts, 3)
+    assert m.pool_bytes(2) == used
+
+
 def test_what_a_token_sees():
     # window of 5, blocks of 3: token 9 sees tokens 5..9 and the block 0..2 (ends at 2 <= 4); block 3..5 ends at 5 > 4
     assert pp.visible(9, 20, 5, 3) == ([0], [5, 6, 7, 8, 9])
