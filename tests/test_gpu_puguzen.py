@@ -546,7 +546,7 @@ def test_unequal_requests_together_with_pages_and_slots_used_again(folders, name
     for rounds in range(2):                      # the second time the steps' shapes are known and recorded
         got = H.run_steps(runner, steps)
         runner.cache.check()
-        compare(got, reqs, folders[name], TOL[dtype], "%s %s mixed, round %d" % (name, dtype, rounds), CLOSE[dtype])
+        compare(got, reqs, folders[name], TOL[dtype], "%s %s mixed, pass %d" % (name, dtype, rounds), CLOSE[dtype])
         if alone is not None:
             for key, row in alone.items():
                 assert np.array_equal(row, got[key]), "%s: in a batch, %s differs from the request alone" % (name, key)
