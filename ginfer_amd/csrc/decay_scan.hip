@@ -7,7 +7,7 @@
 // k_scale.  q, k and v are 32-bit rows of one projection (a common row stride).
 // The state is 32-bit, [slot][head][dim][vdim]; a request whose q_start is 0 starts from zeros.  A workgroup owns one
 // (entry, head, block of 16 value columns) and walks the entry's tokens in order, up to 16 at a time: the tile's q, k, a and v go
-// through LDS, every thread keeps the state of one column and every 16th row in registers, and the rows' partial
+// through LDS (asked for from memory a tile ahead), every thread keeps the state of one column and every 16th row in registers, and the rows' partial
 // outputs are added in a fixed order.  So a token's result does not depend on how the request's tokens were cut into
 // steps, nor on what else is in the batch.
 // gla_decay: a = sigmoid(z)^(1/tau), z = A2 (low) + b (A2 handed over transposed), `low` being the rows of a narrow projection (32-bit), as
@@ -46,10 +46,15 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
   }
   const int hd = heads * dim, half = rot_dims / 2;
   const float hdec = head_decay ? head_decay[h] : 0.f;
-  for (int t0 = 0; t0 < n; t0 += TILE) {
+  // A thread's share of a tile's q, k and a (PER elements each) and one v: asked for a tile ahead, into registers, so
+  // that the way to memory runs beside the walk over the tile before.
+  constexpr int PER = TILE * DP / DS_THREADS;
+  float rq[PER], rk[PER], ra[PER], rv;
+  auto fetch = [&](int t0) {
     const int nt = min(TILE, n - t0);
-    __syncthreads();                                   // the tile before is read out
-    for (int idx = threadIdx.x; idx < TILE * DP; idx += DS_THREADS) {
+#pragma unroll
+    for (int x = 0; x < PER; ++x) {
+      const int idx = threadIdx.x + x * DS_THREADS;
       const int tt = idx / DP, i = idx % DP;
       float qv = 0.f, kv = 0.f, a = 0.f;
       if (tt < nt && i < dim) {
@@ -71,15 +76,30 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
         kv *= k_scale;
         a = decay ? decay[row * hd + h * dim + i] : hdec;
       }
-      qs[tt][i] = qv;
-      ks[tt][i] = kv;
-      as[tt][i] = a;
+      rq[x] = qv;
+      rk[x] = kv;
+      ra[x] = a;
+    }
+    const int tt = threadIdx.x / DS_COLS, jj = threadIdx.x % DS_COLS;      // 16 * DS_COLS == DS_THREADS
+    rv = (tt < nt && v0 + jj < vdim) ? v[(int64_t)(first + t0 + tt) * stride + h * vdim + v0 + jj] : 0.f;
+  };
+  fetch(0);
+  for (int t0 = 0; t0 < n; t0 += TILE) {
+    const int nt = min(TILE, n - t0);
+    __syncthreads();                                   // the tile before is read out
+#pragma unroll
+    for (int x = 0; x < PER; ++x) {
+      const int idx = threadIdx.x + x * DS_THREADS;
+      qs[idx / DP][idx % DP] = rq[x];
+      ks[idx / DP][idx % DP] = rk[x];
+      as[idx / DP][idx % DP] = ra[x];
     }
     {
-      const int tt = threadIdx.x / DS_COLS, jj = threadIdx.x % DS_COLS;      // 16 * DS_COLS == DS_THREADS
-      if (tt < TILE) vs[tt][jj] = (tt < nt && v0 + jj < vdim) ? v[(int64_t)(first + t0 + tt) * stride + h * vdim + v0 + jj] : 0.f;
+      const int tt = threadIdx.x / DS_COLS, jj = threadIdx.x % DS_COLS;
+      if (tt < TILE) vs[tt][jj] = rv;
     }
     __syncthreads();
+    if (t0 + TILE < n) fetch(t0 + TILE);
     for (int tt = 0; tt < nt; ++tt) {
       const float vv = vs[tt][j];
       float acc = 0.f;
