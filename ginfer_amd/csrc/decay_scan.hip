@@ -135,6 +135,7 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
 // widening matrix TRANSPOSED, [rank][channels]: neighbouring threads read neighbouring channels.  A workgroup takes GD_TOKENS
 // tokens and 256 channels; the tokens' narrow rows go through LDS and every element of a2t is read once for all of them.
 #define GD_TOKENS 16
+#define GD_BATCH 32
 __global__ __launch_bounds__(256) void gla_decay_kernel(float* __restrict__ decay, const float* __restrict__ low,
                                                         int64_t low_stride, const float* __restrict__ a2t,
                                                         const float* __restrict__ bias, int tokens, int channels, int rank,
@@ -151,12 +152,12 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(float* __restrict__ deca
   float z[GD_TOKENS];
 #pragma unroll
   for (int tt = 0; tt < GD_TOKENS; ++tt) z[tt] = 0.f;
-  for (int r0 = 0; r0 < rank; r0 += 8) {               // eight elements of a2t are asked for at a time
-    float w[8];
+  for (int r0 = 0; r0 < rank; r0 += GD_BATCH) {        // GD_BATCH elements of a2t are asked for at a time: in a decode step
+    float w[GD_BATCH];                                 // every one comes from memory, a microsecond away
 #pragma unroll
-    for (int j = 0; j < 8; ++j) w[j] = r0 + j < rank ? a2t[(int64_t)(r0 + j) * channels + c] : 0.f;
+    for (int j = 0; j < GD_BATCH; ++j) w[j] = r0 + j < rank ? a2t[(int64_t)(r0 + j) * channels + c] : 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < GD_BATCH; ++j) {
       if (r0 + j < rank) {
         const float* lo = lows + (r0 + j) * GD_TOKENS;
 #pragma unroll

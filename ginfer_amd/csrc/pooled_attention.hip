@@ -108,41 +108,60 @@ __device__ __forceinline__ int64_t pa_row(const int32_t* __restrict__ table, int
   return page < 0 ? -1 : (int64_t)page * page_size + (p - b * page_size);
 }
 
+// The mean over the block that ends at `pos` of one channel: eight rows are asked for at a time, without a branch in
+// between (a row that is not there is read at row 0 and left out), and added in the order of the positions.
+template <bool KEYS, typename TC>
+__device__ __forceinline__ float pa_block_mean(const TC* __restrict__ rows, const int32_t* __restrict__ bt, int width, int pos,
+                                               int pool, int page_size, int nkv, int g, int w, int c) {
+  float sum = 0.f;
+  for (int p0 = pos + 1 - pool; p0 <= pos; p0 += 8) {
+    int page[8], at[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int p = p0 + j <= pos ? p0 + j : pos;
+      const int b = p / page_size;
+      at[j] = p - b * page_size;
+      page[j] = bt[b < width ? b : width - 1];
+      if (b >= width || p0 + j > pos) page[j] = -1;
+    }
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int64_t pg = page[j] < 0 ? 0 : page[j];
+      x[j] = KEYS ? Num<TC>::ld(rows + ((pg * page_size + at[j]) * nkv + g) * (int64_t)w + c)
+                  : Num<TC>::ld(rows + ((pg * nkv + g) * (int64_t)w + c) * page_size + at[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (page[j] >= 0) sum += x[j];
+  }
+  return sum / (float)pool;
+}
+
 // grid (tokens, 2 nkv): the keys' and the values' heads of the block that a token ends
 template <typename TC>
 __global__ __launch_bounds__(256) void pwa_pool_kernel(float* __restrict__ pk_rows, float* __restrict__ pv_rows,
-                                                              const TC* __restrict__ k_rows, const TC* __restrict__ v_rows,
-                                                              const int32_t* __restrict__ positions,
-                                                              const int32_t* __restrict__ token_entry,
-                                                              const int32_t* __restrict__ table, int width,
-                                                              const int64_t* __restrict__ pool_slots, int nkv, int dim, int vdim,
-                                                              int pool, int page_size) {
+                                                       const TC* __restrict__ k_rows, const TC* __restrict__ v_rows,
+                                                       const int32_t* __restrict__ positions,
+                                                       const int32_t* __restrict__ token_entry,
+                                                       const int32_t* __restrict__ table, int width,
+                                                       const int64_t* __restrict__ pool_slots, int nkv, int dim, int vdim,
+                                                       int pool, int page_size) {
   const int64_t t = blockIdx.x;
   const int pos = positions[t];
   if ((pos + 1) % pool) return;
   const int64_t dst_row = pool_slots[t];
   if (dst_row < 0) return;
-  const int e = token_entry[t];
-  const bool keys = blockIdx.y < (unsigned)nkv;
-  const int g = keys ? blockIdx.y : blockIdx.y - nkv, w = keys ? dim : vdim;
-  const float inv = 1.0f / (float)pool;
-  for (int c = threadIdx.x; c < w; c += blockDim.x) {
-    float sum = 0.f;
-    // eight rows are asked for at a time and added in the order of the positions
-    for (int p0 = pos + 1 - pool; p0 <= pos; p0 += 8) {
-      float x[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int64_t r = p0 + j <= pos ? pa_row(table, width, e, p0 + j, page_size) : -1;
-        x[j] = r < 0 ? 0.f : keys ? Num<TC>::ld(k_rows + (r * nkv + g) * (int64_t)w + c)
-                                  : Num<TC>::ld(v_rows + pa_value_at(r, g, c, nkv, vdim, page_size));
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if (p0 + j <= pos) sum += x[j];
-    }
-    if (keys) pk_rows[(dst_row * nkv + g) * (int64_t)w + c] = sum * inv;
-    else pv_rows[pa_value_at(dst_row, g, c, nkv, vdim, page_size)] = sum * inv;
+  const int32_t* bt = table + (int64_t)token_entry[t] * width;
+  if (blockIdx.y < (unsigned)nkv) {
+    const int g = blockIdx.y;
+    for (int c = threadIdx.x; c < dim; c += blockDim.x)
+      pk_rows[(dst_row * nkv + g) * (int64_t)dim + c] = pa_block_mean<true, TC>(k_rows, bt, width, pos, pool, page_size, nkv, g, dim, c);
+  } else {
+    const int g = blockIdx.y - nkv;
+    for (int c = threadIdx.x; c < vdim; c += blockDim.x)
+      pv_rows[pa_value_at(dst_row, g, c, nkv, vdim, page_size)] =
+          pa_block_mean<false, TC>(v_rows, bt, width, pos, pool, page_size, nkv, g, vdim, c);
   }
 }
 
