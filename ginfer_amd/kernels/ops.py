@@ -1332,7 +1332,7 @@ POOLED_ATTENTION_MAX_DIM = 256
 
 
 def _token_rows(t, width, name, dtype=None):
-    """A paged tensor viewed as rows of `width` elements, a slot a row."""
+    """How many slots a paged tensor of `width` elements a slot holds (keys lie a slot a row; values transposed inside a page)."""
     _need(t is not None and t.is_contiguous() and t.numel() % width == 0 and (dtype is None or t.dtype == dtype),
           "%s must be contiguous%s and hold whole rows of %d", name, "" if dtype is None else " " + str(dtype), width)
     return t.numel() // width
@@ -1389,7 +1389,8 @@ def _table(t, entries, name):
 
 def pooled_attention_pool(pk_rows, pv_rows, k_rows, v_rows, step, table, pool_slots, num_kv_heads, dim, vdim, pool, page_size):
     """For every token of the step that ends a block of `pool` positions: the means of the block's cached keys and values
-    (read through the entries' block `table`) into the float32 rows pk_rows, pv_rows at pool_slots[token] (-1: none)."""
+    (read through the entries' block `table`) into the float32 pages pk_rows, pv_rows (laid out as the tokens' pages, a block for
+    a token) at pool_slots[token] (-1: none)."""
     _dev(pk_rows, pv_rows, k_rows, v_rows, table, pool_slots)
     T = step.positions.shape[0]
     E = step.cu_tokens.shape[0] - 1
@@ -1410,8 +1411,9 @@ def pooled_attention_pool(pk_rows, pv_rows, k_rows, v_rows, step, table, pool_sl
 
 def pooled_attention(q, k_rows, v_rows, pk_rows, pv_rows, step, table, pool_table, head_bias, num_heads, num_kv_heads, dim, vdim,
                      size, pool, page_size, scale, dtype, proj=None, gate_start=0):
-    """q float32 [T, num_heads * dim].  Token i sees the tokens j with 0 <= i - j < size and the means of the blocks of `pool`
-    tokens that end before them; the weight of a key is sigmoid(scale q . k + head_bias[head]) (head_bias float32 [heads] or
+    """q float32 [T, num_heads * dim]; k_rows, v_rows: the tokens' pages (keys [page][slot][kv head][dim], values [page][kv head][vdim]
+    [slot]), pk_rows, pv_rows: the blocks' means, float32, laid out alike.  Token i sees the tokens j with 0 <= i - j < size and the
+    means of the blocks of `pool` tokens that end before them; the weight of a key is sigmoid(scale q . k + head_bias[head]) (head_bias float32 [heads] or
     None), not normalised.  The result is multiplied by sigmoid of the gate, the columns gate_start .. of the float32 projection
     `proj` (None: no gate).  Returns [T, num_heads * vdim] in `dtype`."""
     _dev(q, k_rows, v_rows, pk_rows, pv_rows, table, pool_table, head_bias, proj)
