@@ -1,5 +1,5 @@
 // Sublayers that run side by side and enter the residual stream through gates of their own:
-//   residual[t] += sigmoid(z1[t]) * y1[t] (+ sigmoid(z2[t]) * y2[t])         z: 32-bit rows [tokens, gates * hidden]
+//   residual[t] += sigmoid(z1[t]) * y1[t] (+ sigmoid(z2[t]) * y2[t])         z: 32-bit rows of gates * hidden numbers with a stride
 //   next[t]      = g * residual[t] / sqrt(mean(residual[t]^2) + eps)         (optional: the norm that is read next)
 // The gated results are added to each other first and then to the stream.  All arithmetic in 32-bit; a row's sum of
 // squares is taken in an order that depends on its length alone.  A workgroup a token.
@@ -14,11 +14,11 @@ template <typename Y, typename C>
 __global__ __launch_bounds__(GRS_THREADS) void gated_residual_add_kernel(float* __restrict__ residual, const float* __restrict__ z,
                                                                           const Y* __restrict__ y1, const Y* __restrict__ y2,
                                                                           const float* __restrict__ next_gain, float next_eps,
-                                                                          C* __restrict__ next, int hidden) {
+                                                                          C* __restrict__ next, int hidden, int64_t z_stride) {
   __shared__ float scratch[GRS_THREADS / WAVE];
   const int64_t t = blockIdx.x;
   float* res = residual + t * hidden;
-  const float* zr = z + t * (int64_t)hidden * (y2 ? 2 : 1);
+  const float* zr = z + t * z_stride;
   const Y* a = y1 + t * hidden;
   const Y* b = y2 ? y2 + t * hidden : nullptr;
   float ss = 0.f;
@@ -61,11 +61,11 @@ template <typename Y, typename C, int PER>
 __global__ __launch_bounds__(GRS_THREADS) void gated_residual_add_quad_kernel(float* __restrict__ residual, const float* __restrict__ z,
                                                                                const Y* __restrict__ y1, const Y* __restrict__ y2,
                                                                                const float* __restrict__ next_gain, float next_eps,
-                                                                               C* __restrict__ next, int hidden) {
+                                                                               C* __restrict__ next, int hidden, int64_t z_stride) {
   __shared__ float scratch[GRS_THREADS / WAVE];
   const int64_t t = blockIdx.x;
   float* res = residual + t * hidden;
-  const float* zr = z + t * (int64_t)hidden * (y2 ? 2 : 1);
+  const float* zr = z + t * z_stride;
   const Y* a = y1 + t * hidden;
   const Y* b = y2 ? y2 + t * hidden : nullptr;
   float4 r[PER], za[PER], zb[PER], ya[PER], yb[PER];
@@ -113,16 +113,16 @@ __global__ __launch_bounds__(GRS_THREADS) void gated_residual_add_quad_kernel(fl
   }
 }
 
-extern "C" int ga_gated_residual_add(void* residual, const void* z, const void* y1, const void* y2, int tokens, int hidden,
+extern "C" int ga_gated_residual_add(void* residual, const void* z, int64_t z_stride, const void* y1, const void* y2, int tokens, int hidden,
                                      int y_bf16, const void* next_gain, float next_eps, void* next, int next_bf16,
                                      hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (hidden <= 0 || !z || !y1 || ((next != nullptr) != (next_gain != nullptr))) return -1;
   dim3 grid(tokens), block(GRS_THREADS);
-  if (hidden % 4 == 0 && hidden <= GRS_THREADS * 4 * 8) {
+  if (hidden % 4 == 0 && hidden <= GRS_THREADS * 4 * 8 && z_stride % 4 == 0 && ((uintptr_t)z & 15) == 0) {
 #define GQ(Y, C, PER) hipLaunchKernelGGL((gated_residual_add_quad_kernel<Y, C, PER>), grid, block, 0, stream, (float*)residual,   \
                                          (const float*)z, (const Y*)y1, (const Y*)y2, (const float*)next_gain, next_eps, (C*)next, \
-                                         hidden)
+                                         hidden, z_stride)
 #define GP(Y, C) do { if (hidden <= GRS_THREADS * 4) GQ(Y, C, 1); else if (hidden <= GRS_THREADS * 8) GQ(Y, C, 2);              \
                       else if (hidden <= GRS_THREADS * 16) GQ(Y, C, 4); else GQ(Y, C, 8); } while (0)
     if (y_bf16) { if (next_bf16) GP(bf16_t, bf16_t); else GP(bf16_t, float); }
@@ -133,7 +133,7 @@ extern "C" int ga_gated_residual_add(void* residual, const void* z, const void* 
   }
 #define GO(Y, C) hipLaunchKernelGGL((gated_residual_add_kernel<Y, C>), grid, block, 0, stream, (float*)residual,          \
                                     (const float*)z, (const Y*)y1, (const Y*)y2, (const float*)next_gain, next_eps, (C*)next, \
-                                    hidden)
+                                    hidden, z_stride)
   if (y_bf16) { if (next_bf16) GO(bf16_t, bf16_t); else GO(bf16_t, float); }
   else { if (next_bf16) GO(float, bf16_t); else GO(float, float); }
 #undef GO

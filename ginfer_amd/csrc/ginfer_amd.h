@@ -273,8 +273,9 @@ int ga_pwa_attend_mfma(void* out, void* partial, const void* q, const void* k_ro
                        int page_size, float scale, hipStream_t stream);
 
 // ---- gated_residual.hip: residual float [tokens, hidden] += sigmoid(z[:, :hidden]) * y1 (+ sigmoid(z[:, hidden:]) * y2, y2
-// may be null); with next: next = rmsnorm(residual) * next_gain (float [hidden])
-int ga_gated_residual_add(void* residual, const void* z, const void* y1, const void* y2, int tokens, int hidden, int y_bf16,
+// may be null; z: float rows with the stride z_stride); with next: next = rmsnorm(residual) * next_gain (float [hidden])
+int ga_gated_residual_add(void* residual, const void* z, int64_t z_stride, const void* y1, const void* y2, int tokens, int hidden,
+                          int y_bf16,
                           const void* next_gain, float next_eps, void* next, int next_bf16, hipStream_t stream);
 
 // ---- random_fill.hip: out[i] = mean + std * normal(key, i) for n elements, float or bfloat16: the counter-based

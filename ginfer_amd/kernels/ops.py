@@ -1469,13 +1469,15 @@ def pooled_attention(q, k_rows, v_rows, pk_rows, pv_rows, step, table, pool_tabl
 
 def gated_residual_add(residual, z, y1, y2=None, next_gain=None, next_eps=0.0, dtype=None):
     """residual float32 [T, H] += sigmoid(z[:, :H]) * y1 (+ sigmoid(z[:, H:]) * y2), the gated results added to each other
-    first; z float32 [T, H] or [T, 2H]; y1, y2 [T, H] in float32 or bfloat16.  With next_gain (float32 [H]) the rows of the norm
+    first; z float32 [T, H] or [T, 2H] (rows may have a stride: columns of a wider projection); y1, y2 [T, H] in float32 or
+    bfloat16.  With next_gain (float32 [H]) the rows of the norm
     that is read next, rmsnorm(residual) * next_gain in `dtype`, come back; else None."""
     _dev(residual, z, y1, y2, next_gain)
     _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(), "residual must be contiguous float32 [T, H]")
     T, H = residual.shape
     gates = 1 if y2 is None else 2
-    _f32(z, (T, gates * H), "z")
+    _need(z.dtype == torch.float32 and tuple(z.shape) == (T, gates * H) and z.stride(1) == 1,
+          "z must be float32 [%d, %d] with unit inner stride (it may be columns of a wider projection)", T, gates * H)
     for name, y in (("y1", y1), ("y2", y2)):
         _need(y is None or (y.shape == (T, H) and y.is_contiguous() and y.dtype == y1.dtype), "%s must be contiguous [%d, %d] in one dtype", name, T, H)
     nxt = None
@@ -1483,7 +1485,7 @@ def gated_residual_add(residual, z, y1, y2=None, next_gain=None, next_eps=0.0, d
         _f32(next_gain, (H,), "next_gain")
         nxt = torch.empty((T, H), dtype=dtype, device=residual.device)
     lib = build.load("gated_residual")
-    _check(lib.ga_gated_residual_add(_ptr(residual), _ptr(z), _ptr(y1), _ptr(y2), _i(T), _i(H), _i(_is_bf16(y1.dtype)),
+    _check(lib.ga_gated_residual_add(_ptr(residual), _ptr(z), _i64(z.stride(0)), _ptr(y1), _ptr(y2), _i(T), _i(H), _i(_is_bf16(y1.dtype)),
                                      _ptr(next_gain), _f(next_eps), _ptr(nxt), _i(_is_bf16(dtype) if nxt is not None else 0),
                                      _stream()), "gated_residual_add")
     return nxt

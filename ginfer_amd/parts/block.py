@@ -204,7 +204,8 @@ class ParallelGatedBlock(Arrangement):
     """n = norm(x);  x <- x + (gate1(n) * mixer(n) + gate2(n) * feed_forward(n)): ONE norm, both sublayers read its rows side
     by side, and each result enters the stream through a gate that reads the same rows (a part of the `residual_gate`
     family: `logits(n)`, `add(residual, z, results, then)`).  A layer may have no feed-forward (its gate part then names one
-    gate).  The 32-bit stream is updated in place; where the model hands over the norm of the block that runs next
+    gate).  Where the gate part can hand its matrix to the mixer (`hand_over`; the mixer has `append_columns`), the gates'
+    logits come out of the mixer's own projection: both read the same rows.  The 32-bit stream is updated in place; where the model hands over the norm of the block that runs next
     (`into_norm`), the launch that adds the results also makes that norm's rows (the next block then gets `NormedRows` in
     place of a delta)."""
 
@@ -216,6 +217,7 @@ class ParallelGatedBlock(Arrangement):
     def __init__(self, parts):
         super().__init__(parts)
         self.feed_forward = self._parts.get("feed_forward")
+        self._one_product = None
         gates = len(getattr(self.gate, "names", ()))
         if gates != (1 if self.feed_forward is None else 2):
             raise ValueError("a block gates each of its sublayers: %d gates for %d sublayers"
@@ -230,8 +232,15 @@ class ParallelGatedBlock(Arrangement):
             n = delta.rows
         else:
             n = self.norm.forward(residual, whole(delta, self.norm))
-        z = self.gate.logits(n)
-        results = [self.mixer.forward(n, step, cache)]
+        if self._one_product is None:           # once the weights are bound: the gates' matrix behind the mixer's own projection
+            hand = getattr(self.gate, "hand_over", None)
+            self._one_product = bool(hand is not None and hand(self.mixer))
+        if self._one_product:
+            results = [self.mixer.forward(n, step, cache)]
+            z = self.mixer.extra_columns
+        else:
+            z = self.gate.logits(n)
+            results = [self.mixer.forward(n, step, cache)]
         if self.feed_forward is not None:
             results.append(self.feed_forward.forward(n))
         rows = self.gate.add(residual, z, [whole(r).to(n.dtype) if r.dim() == 3 else r for r in results], then=into_norm)

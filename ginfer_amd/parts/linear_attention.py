@@ -24,10 +24,24 @@ class _DecayedLinearAttention(Part):
                              % (key_dim, ops.DECAY_SCAN_MAX_DIM))
         self.hidden_size, self.nh, self.dk, self.dv = int(hidden_size), int(num_heads), int(key_dim), int(value_dim)
         self.eps, self.dtype, self.device = float(eps), dtype, device
-        self.w_in = self.w_o = None
+        self.w_in = self.w_o = self.b_in = self._extra = self.extra_columns = None
 
     def cache_spec(self):
         return StateSpec((self.nh, self.dk, self.dv), torch.float32)
+
+    # Columns that someone else wants of the same rows (a block's gates read what the mixer reads): their matrix is
+    # stacked behind the mixer's own, so that ONE product makes both; forward leaves them in `extra_columns`.
+    def append_columns(self, weight, bias):
+        own = self.w_in.shape[0]
+        self._extra = (own, own + weight.shape[0])
+        self.w_in = torch.cat([self.w_in, weight], dim=0).contiguous()
+        self.b_in = torch.cat([torch.zeros((own,), dtype=bias.dtype, device=bias.device), bias]).contiguous()
+        return True
+
+    def _project(self, x):
+        proj = linear(x, self.w_in, self.b_in, out_dtype=torch.float32)
+        self.extra_columns = proj[:, self._extra[0]:self._extra[1]] if self._extra is not None else None
+        return proj
 
     def _projection_specs(self):
         H, k, v = self.hidden_size, self.nh * self.dk, self.nh * self.dv
@@ -83,7 +97,7 @@ class GatedLinearAttention(_DecayedLinearAttention):
         self.w_o = t["o"]
 
     def forward(self, x, step, cache):
-        proj = linear(x, self.w_in, None, out_dtype=torch.float32)
+        proj = self._project(x)
         decay = ops.gla_decay(proj, self._rest0, self.w_a2, self.b_a2, self.tau)
         o = ops.decay_scan(proj, 0, self._k0, self._v0, cache.state, cache.slots, step, self.nh, self.dk, self.dv,
                            decay=decay, q_scale=self.dk ** -0.5)
@@ -116,7 +130,7 @@ class Retention(_DecayedLinearAttention):
         self.head_decay = torch.tensor(self.decay, dtype=torch.float32, device=self.w_in.device)
 
     def forward(self, x, step, cache):
-        proj = linear(x, self.w_in, None, out_dtype=torch.float32)
+        proj = self._project(x)
         cos, sin = self.position.tables() if self.position is not None else (None, None)
         o = ops.decay_scan(proj, 0, self._k0, self._v0, cache.state, cache.slots, step, self.nh, self.dk, self.dv,
                            head_decay=self.head_decay, cos=cos, sin=sin, k_scale=self.dk ** -0.5)

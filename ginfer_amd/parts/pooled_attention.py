@@ -42,7 +42,7 @@ class PooledWindowAttention(Part):
         self.scale, self.eps = float(scale), float(eps)
         self.unit_norm, self.has_bias, self.gated = bool(unit_norm), bool(head_bias), bool(gated)
         self.dtype, self.device = dtype, device
-        self.w_in = self.w_o = self.head_bias = None
+        self.w_in = self.w_o = self.head_bias = self.b_in = self._extra = self.extra_columns = None
 
     def cache_spec(self):
         """[keys and values of the tokens a query or a block's mean can still need, the blocks' means]."""
@@ -65,6 +65,15 @@ class PooledWindowAttention(Part):
         self.head_bias = t["pb"].float().contiguous() if self.has_bias else None
         self.w_o = t["o"]
 
+    def append_columns(self, weight, bias):
+        """Columns that someone else wants of the same rows (a block's gates): stacked behind the part's own matrix, so that
+        one product makes both; forward leaves them in `extra_columns`."""
+        own = self.w_in.shape[0]
+        self._extra = (own, own + weight.shape[0])
+        self.w_in = torch.cat([self.w_in, weight], dim=0).contiguous()
+        self.b_in = torch.cat([torch.zeros((own,), dtype=bias.dtype, device=bias.device), bias]).contiguous()
+        return True
+
     def kernel_modules(self):
         return ["pooled_attention", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
 
@@ -72,7 +81,8 @@ class PooledWindowAttention(Part):
         near, means = cache
         k_rows, v_rows = near.pages["k"], near.pages["v"]
         pk_rows, pv_rows = means.pages["k"], means.pages["v"]
-        proj = linear(x, self.w_in, None, out_dtype=torch.float32)
+        proj = linear(x, self.w_in, self.b_in, out_dtype=torch.float32)
+        self.extra_columns = proj[:, self._extra[0]:self._extra[1]] if self._extra is not None else None
         cos, sin = self.position.tables() if self.position is not None else (None, None)
         q = ops.pooled_attention_prepare(proj, step.positions, cos, sin, near.slot_mapping, k_rows, v_rows, self.nh, self.nkv,
                                          self.hd, self.vd, self.eps, near.page_size, unit_norm=self.unit_norm, write=near.owner)

@@ -42,7 +42,19 @@ class SigmoidProjectionGate(Part):
 
     def logits(self, x):
         """float32 [T, gates * H]: what the sigmoids are taken of."""
+        if self.weight is None:
+            raise RuntimeError("the gates' matrix was handed to the part that reads the same rows: take its extra columns")
         return linear(x, self.weight, self.bias, out_dtype=torch.float32)
+
+    def hand_over(self, taker):
+        """Gives the gates' matrix and bias to a part that reads the same rows and can stack them behind its own projection
+        (`append_columns(weight, bias)`; its forward then leaves the logits in `extra_columns`).  True if it took them: this
+        part then keeps no copy."""
+        take = getattr(taker, "append_columns", None)
+        if take is None or self.weight is None or not take(self.weight, self.bias):
+            return False
+        self.weight = self.bias = None
+        return True
 
     def add(self, residual, z, results, then=None):
         """residual += sum_i sigmoid(z_i) * results[i] (the gated results added to each other first).  then: a norm with a
