@@ -24,7 +24,7 @@ __global__ __launch_bounds__(GRS_THREADS) void gated_residual_add_kernel(float* 
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += GRS_THREADS) {
     float d = grs_sigmoid(zr[i]) * Num<Y>::ld(a + i);
-    if (b) d += grs_sigmoid(zr[hidden + i]) * Num<Y>::ld(b + i);
+    if (b) d = fmaf(grs_sigmoid(zr[hidden + i]), Num<Y>::ld(b + i), d);
     const float r = res[i] + d;
     res[i] = r;
     ss += r * r;
@@ -90,10 +90,10 @@ __global__ __launch_bounds__(GRS_THREADS) void gated_residual_add_quad_kernel(fl
       float4 d = make_float4(grs_sigmoid(za[j].x) * ya[j].x, grs_sigmoid(za[j].y) * ya[j].y, grs_sigmoid(za[j].z) * ya[j].z,
                              grs_sigmoid(za[j].w) * ya[j].w);
       if (b) {
-        d.x += grs_sigmoid(zb[j].x) * yb[j].x;
-        d.y += grs_sigmoid(zb[j].y) * yb[j].y;
-        d.z += grs_sigmoid(zb[j].z) * yb[j].z;
-        d.w += grs_sigmoid(zb[j].w) * yb[j].w;
+        d.x = fmaf(grs_sigmoid(zb[j].x), yb[j].x, d.x);
+        d.y = fmaf(grs_sigmoid(zb[j].y), yb[j].y, d.y);
+        d.z = fmaf(grs_sigmoid(zb[j].z), yb[j].z, d.z);
+        d.w = fmaf(grs_sigmoid(zb[j].w), yb[j].w, d.w);
       }
       r[j] = make_float4(r[j].x + d.x, r[j].y + d.y, r[j].z + d.z, r[j].w + d.w);
       Quad<float>::st(res + i, r[j]);

@@ -513,6 +513,29 @@ def test_whole_decoded_and_in_portions(folders, name, dtype):
     assert not runner.cache.requests and all(g.pool.num_free == g.pool.num_pages for g in runner.cache.groups)
 
 
+def test_gates_from_the_mixers_projection_or_from_a_product_of_their_own(folders, monkeypatch):
+    """A block's gates ride behind the mixer's projection where the mixer takes their matrix; a mixer that declines leaves
+    them a product of their own.  The same logits within the rounding of 32-bit sums."""
+    from ginfer_amd.parts.linear_attention import GatedLinearAttention, Retention
+    from ginfer_amd.parts.pooled_attention import PooledWindowAttention
+    reqs = requests_for("mix", [33, 70])
+    for dtype in ("float32", "bfloat16"):
+        together = runner_for(folders["mix"], "mix", dtype)
+        got = H.run_steps(together, H.steps_portions(reqs))
+        assert all(b._one_product is True and b.gate.weight is None and b.mixer.extra_columns is not None for b in together.model.blocks)
+        with monkeypatch.context() as m:
+            for cls in (GatedLinearAttention, Retention, PooledWindowAttention):
+                m.setattr(cls, "append_columns", lambda self, weight, bias: False)
+            apart = runner_for(folders["mix"], "mix", dtype)
+            want = H.run_steps(apart, H.steps_portions(reqs))
+            assert all(b._one_product is False and b.gate.weight is not None for b in apart.model.blocks)
+        for key, row in want.items():
+            if dtype == "float32":      # two products or one: other kernels for other sizes, the same numbers within rounding
+                assert H.rel_err(got[key], row) < 2e-6, key
+        compare(got, reqs, folders["mix"], TOL[dtype], "gates with the mixer, " + dtype, CLOSE[dtype])
+        compare(want, reqs, folders["mix"], TOL[dtype], "gates apart, " + dtype, CLOSE[dtype])
+
+
 def test_the_stream_after_every_layer(folders):
     name = "mix"
     ids = H.random_tokens(37, CONFIGS[name][0]["vocab"], 5)
