@@ -5,7 +5,8 @@ from .qwen2 import Qwen2Config
 from .titozen import TitozenConfig
 from .potupel import PotupelConfig
 from .puguzen import PuguzenConfig
+from .nidasun import NidasunConfig
 
 __all__ = ["ConfigError", "register_architecture", "registered_architectures", "config_class",
            "config_from_dict", "config_from_folder", "PartSpec", "LayerSpec", "prenorm_layer", "ScheduleEntry",
-           "ModelSpec", "Qwen2Config", "TitozenConfig", "PotupelConfig", "PuguzenConfig"]
+           "ModelSpec", "Qwen2Config", "TitozenConfig", "PotupelConfig", "PuguzenConfig", "NidasunConfig"]

@@ -83,6 +83,9 @@ class ModelSpec:
     # tail_enter: passes that start behind the last run (a repeated group without layers at the model's end)
     reentry: Optional[PartSpec] = None
     tail_enter: tuple = ()
+    # how the residual stream is kept where it is not one tensor (a part of the `stream` family: several streams side by
+    # side, opened behind the embedding and closed in front of the final norm), or None
+    stream: Optional[PartSpec] = None
 
     def name_of(self, role):
         return self.names.get(role, role)

@@ -210,3 +210,32 @@ extern "C" int ga_relu_square(void* out, const void* x, int64_t total, int is_bf
   else hipLaunchKernelGGL(relu_square_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)x, total);
   return GA_CHECK_LAUNCH();
 }
+
+// Two results side by side, each with a factor: out[i] = sa * a[i] + sb * b[i], in 32-bit.  out may be a or b.
+template <typename T>
+__global__ __launch_bounds__(256) void scaled_sum_kernel(T* __restrict__ out, const T* __restrict__ a, const T* __restrict__ b,
+                                                         float sa, float sb, int64_t total) {
+  constexpr int V = 16 / sizeof(T);
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+  if (i + V <= total) {
+    union { uint4 u; T e[V]; } x, y, o;
+    x.u = *reinterpret_cast<const uint4*>(a + i);
+    y.u = *reinterpret_cast<const uint4*>(b + i);
+#pragma unroll
+    for (int j = 0; j < V; ++j) Num<T>::st(&o.e[j], fmaf(sb, Num<T>::ld(&y.e[j]), sa * Num<T>::ld(&x.e[j])));
+    *reinterpret_cast<uint4*>(out + i) = o.u;
+  } else {
+    for (int64_t k = i; k < total; ++k) Num<T>::st(out + k, fmaf(sb, Num<T>::ld(b + k), sa * Num<T>::ld(a + k)));
+  }
+}
+
+extern "C" int ga_scaled_sum(void* out, const void* a, const void* b, float sa, float sb, int64_t total, int is_bf16,
+                             hipStream_t stream) {
+  if (total <= 0) return 0;
+  if (((uintptr_t)out | (uintptr_t)a | (uintptr_t)b) % 16) return -1;
+  const int v = is_bf16 ? 8 : 4;
+  dim3 grid((unsigned)((total + 256 * v - 1) / (256 * v))), block(256);
+  if (is_bf16) hipLaunchKernelGGL(scaled_sum_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)a, (const bf16_t*)b, sa, sb, total);
+  else hipLaunchKernelGGL(scaled_sum_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)a, (const float*)b, sa, sb, total);
+  return GA_CHECK_LAUNCH();
+}

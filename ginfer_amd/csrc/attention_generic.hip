@@ -93,7 +93,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
   const int64_t t = t0 + tl;
   const bool live = wave < waves && t < tokens && hl < group;
   const int pos = live ? positions[t] : -1;
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = first_visible_key(pos, window);
   if (live) {
     const T* qp = q + t * q_stride + (int64_t)h * hd;
     for (int d = lane; d < hd; d += WAVE) q_s[wave * hd + d] = Num<T>::ld(qp + d);
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
     int run_end = run_begin, lo_min = 0x7fffffff, pos_max = -1;
     while (run_end < tq && t0 + run_end < tokens && token_entry[t0 + run_end] == run_entry) {
       const int p = positions[t0 + run_end];
-      const int l0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+      const int l0 = first_visible_key(p, window);
       lo_min = l0 < lo_min ? l0 : lo_min;
       pos_max = p > pos_max ? p : pos_max;
       ++run_end;
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
   const int64_t t = t0 + tl;
   const bool live = !loader && hl < group && t < tokens;
   const int pos = live ? positions[t] : -1;
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = first_visible_key(pos, window);
   const int ltid = (int)threadIdx.x - waves * WAVE;          // a loading thread's number
   // The workgroup's tokens from `begin` on that are of one request: the run's end, and the range of keys that its
   // tokens see.  Loaders and the others walk the same runs and tiles, and meet at the same barriers.
@@ -477,7 +477,7 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
     Run r{token_entry[t0 + begin], begin, 0x7fffffff, -1, run_is_shorter(token_entry, t0 + begin, tokens, MA_MIN_RUN)};
     while (r.end < span && t0 + r.end < tokens && token_entry[t0 + r.end] == r.entry) {
       const int p = positions[t0 + r.end];
-      const int l0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+      const int l0 = first_visible_key(p, window);
       r.lo_min = l0 < r.lo_min ? l0 : r.lo_min;
       r.pos_max = p > r.pos_max ? p : r.pos_max;
       ++r.end;
@@ -686,7 +686,7 @@ __global__ __launch_bounds__(64 * (HA_COMPUTE + HA_LOADERS)) void paged_attentio
   const int g = blockIdx.y / head_blocks, hl = (blockIdx.y % head_blocks) * 16 + col;
   const int h = g * group + hl;
   const int pos = positions[t];
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = first_visible_key(pos, window);
   if (wave >= HA_COMPUTE) {
     const TileLoader<T, VEC, HD, HA_LOADERS> loading{k_pages, v_pages, block_table + (int64_t)token_entry[t] * table_width,
                                                      nkv, g, page_size, lo, pos, (int)threadIdx.x - HA_COMPUTE * WAVE,

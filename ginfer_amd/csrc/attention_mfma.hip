@@ -416,7 +416,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
   const int group = nh / nkv;
   const int4 info = decode_info[ti];       // (row of the step, position, entry of the block table, -): one load
   const int t = info.x, pos = info.y;
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = first_visible_key(pos, window);
   const bool col_ok = hb * 16 + c < group;
   const int head = kvh * group + hb * 16 + c;
 
@@ -639,7 +639,7 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
   const int head = kvh * group + hb * hpw + hl;
   const int32_t* tile = tiles + (int64_t)bx * 4;
   const int entry = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
-  const int kv_min_t = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int kv_min_t = first_visible_key(pos0, window);
   const KeyPart kp = key_part(parts, bx, (kv_min_t / 32) * 32, ((pos0 + rows - 1) / 32 + 1) * 32);
 
   f32x4 o[NB][DB];
@@ -653,13 +653,13 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
       const int j = nb * 16 + c;
       const bool ok = j < rows;
       cpos[nb] = ok ? pos0 + j : -1;
-      clo[nb] = (window > 0 && pos0 + j - window + 1 > 0) ? pos0 + j - window + 1 : 0;
+      clo[nb] = first_visible_key(pos0 + j, window);
       load_q(qr[nb], ok ? q + (int64_t)(row0 + j) * q_stride + (int64_t)head * HD : nullptr, g);
     }
-    const int kv_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    const int kv_min = first_visible_key(pos0, window);
     const int kv_max = pos0 + rows - 1;
     // every row of the tile sees the keys from the last row's window start up to the first row's position
-    const int full_lo = (window > 0 && kv_max - window + 1 > 0) ? kv_max - window + 1 : 0;
+    const int full_lo = first_visible_key(kv_max, window);
     attend_tiles<NB, PREFILL_DEPTH>(o, m, l, qr, cpos, clo, k_pages, v_pages,
                                     block_table + (int64_t)__builtin_amdgcn_readfirstlane(entry) * table_width,
                                     table_width, kvh, nkv, ps_shift, kv_min, kv_max, full_lo, pos0,
@@ -809,10 +809,10 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_shared_kernel
   const int32_t* tile = tiles + (int64_t)bx * 4;
   const int entry = __builtin_amdgcn_readfirstlane(tile[0]), row0 = __builtin_amdgcn_readfirstlane(tile[1]),
             rows = __builtin_amdgcn_readfirstlane(tile[2]), pos0 = __builtin_amdgcn_readfirstlane(tile[3]);
-  const int kv_min = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int kv_min = first_visible_key(pos0, window);
   const int kv_max = pos0 + rows - 1;
   // every row of the tile sees the keys from the last row's window start up to the first row's position
-  const int full_lo = (window > 0 && kv_max - window + 1 > 0) ? kv_max - window + 1 : 0;
+  const int full_lo = first_visible_key(kv_max, window);
   const KeyPart kp = key_part(parts, bx, (kv_min / 32) * 32, (kv_max / 32 + 1) * 32);
   const int first = kp.begin, tile_end = kp.end, stride = 32 * splits;
   const int iterations = (tile_end - first + stride - 1) / stride;       // of stream 0, the longest
@@ -860,7 +860,7 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_shared_kernel
       const int j = nb * 16 + c;
       const bool ok = head_ok && j < rows;
       cpos[nb] = ok ? pos0 + j : -1;
-      clo[nb] = (window > 0 && pos0 + j - window + 1 > 0) ? pos0 + j - window + 1 : 0;
+      clo[nb] = first_visible_key(pos0 + j, window);
       load_q(qr[nb], ok ? q + (int64_t)(row0 + j) * q_stride + (int64_t)head * HD : nullptr, g);
     }
     // where this lane's operands lie in a stage: the two key rows of its products, piece by piece, and its values

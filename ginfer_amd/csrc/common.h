@@ -57,6 +57,17 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return t;
 }
 
+// The first key that a query at position `pos` sees, by the kernels' one mask parameter `window`:
+//   window > 0   a sliding window: the keys pos - window + 1 .. pos
+//   window < 0   chunks of -window positions counted from position 0: the keys of pos's own chunk up to pos
+//   window == 0  every key up to pos
+// Both bounds never fall as pos grows, which is what the tiles' shortcuts rely on.
+__host__ __device__ __forceinline__ int first_visible_key(int pos, int window) {
+  if (window > 0) return pos - window + 1 > 0 ? pos - window + 1 : 0;
+  if (window < 0) return pos - pos % (-window);
+  return 0;
+}
+
 #define GA_CHECK_LAUNCH() ((int)hipGetLastError())
 
 // Page and place in the page of a cache slot (slot >= 0).  Page sizes are powers of two nearly always: then a shift,

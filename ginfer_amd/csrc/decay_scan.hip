@@ -12,7 +12,8 @@
 // steps, nor on what else is in the batch.
 // gla_decay: a = sigmoid(z)^(1/tau), z = A2 (low) + b (A2 handed over transposed), `low` being the rows of a narrow projection (32-bit), as
 //   exp(-softplus(-z) / tau), all in 32-bit.
-// head_norm_gate: out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) (* weight[:]) (* silu(gate[t, h, :])).
+// head_norm_gate: out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) (* weight[:]) (* silu(gate[t, h, :]), or * sigmoid of it).
+// silu_inputs: the recurrence reads silu(q), silu(k), silu(v) in place of the projection's numbers.
 #include "common.h"
 #include "ginfer_amd.h"
 
@@ -26,7 +27,7 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
     int64_t stride, const float* __restrict__ decay, const float* __restrict__ head_decay, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int rot_dims, float q_scale, float k_scale, float* __restrict__ state,
     const int64_t* __restrict__ slots, const int32_t* __restrict__ cu, const int32_t* __restrict__ q_start, int heads,
-    int dim, int vdim) {
+    int dim, int vdim, int silu_inputs) {
   constexpr int DP = DS_SLICES * R;
   __shared__ float qs[TILE][DP], ks[TILE][DP], as[TILE][DP], vs[TILE][DS_COLS];
   __shared__ float partial[TILE][DS_SLICES][DS_COLS];
@@ -50,6 +51,8 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
   // that the way to memory runs beside the walk over the tile before.
   constexpr int PER = TILE * DP / DS_THREADS;
   float rq[PER], rk[PER], ra[PER], rv;
+  // q, k and v as the recurrence reads them: the projection's numbers, or their silu
+  auto act = [&](float z) { return silu_inputs ? z / (1.0f + expf(-z)) : z; };
   auto fetch = [&](int t0) {
     const int nt = min(TILE, n - t0);
 #pragma unroll
@@ -61,13 +64,13 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
         const int64_t row = first + t0 + tt;
         const float* qp = q + row * stride + h * dim;
         const float* kp = k + row * stride + h * dim;
-        qv = qp[i];
-        kv = kp[i];
+        qv = act(qp[i]);
+        kv = act(kp[i]);
         if (i < rot_dims) {
           const int f = i < half ? i : i - half, other = i < half ? i + half : i - half;
           const int64_t at = (int64_t)(start + t0 + tt) * half + f;
           const float c = cos_t[at], sn = sin_t[at];
-          const float qo = qp[other], ko = kp[other];
+          const float qo = act(qp[other]), ko = act(kp[other]);
           // the pair (lo, hi) becomes (lo c - hi s, hi c + lo s)
           qv = i < half ? qv * c - qo * sn : qv * c + qo * sn;
           kv = i < half ? kv * c - ko * sn : kv * c + ko * sn;
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
       ra[x] = a;
     }
     const int tt = threadIdx.x / DS_COLS, jj = threadIdx.x % DS_COLS;      // 16 * DS_COLS == DS_THREADS
-    rv = (tt < nt && v0 + jj < vdim) ? v[(int64_t)(first + t0 + tt) * stride + h * vdim + v0 + jj] : 0.f;
+    rv = (tt < nt && v0 + jj < vdim) ? act(v[(int64_t)(first + t0 + tt) * stride + h * vdim + v0 + jj]) : 0.f;
   };
   fetch(0);
   for (int t0 = 0; t0 < n; t0 += TILE) {
@@ -182,7 +185,8 @@ template <typename T>
 __global__ __launch_bounds__(DS_THREADS) void head_norm_gate_kernel(T* __restrict__ out, const float* __restrict__ x,
                                                                      const float* __restrict__ weight,
                                                                      const float* __restrict__ gate, int64_t gate_stride,
-                                                                     int64_t rows, int heads, int vdim, float eps) {
+                                                                     int64_t rows, int heads, int vdim, float eps,
+                                                                     int sigmoid_gate, int weight_per_head) {
   const int64_t row = (int64_t)blockIdx.x * (DS_THREADS / WAVE) + threadIdx.x / WAVE;
   if (row >= rows) return;
   const int lane = threadIdx.x % WAVE;
@@ -196,10 +200,10 @@ __global__ __launch_bounds__(DS_THREADS) void head_norm_gate_kernel(T* __restric
   const float* g = gate ? gate + t * gate_stride + (int64_t)h * vdim : nullptr;
   for (int i = lane; i < vdim; i += WAVE) {
     float y = p[i] / rms;
-    if (weight) y *= weight[i];
+    if (weight) y *= weight[weight_per_head ? (int64_t)h * vdim + i : i];
     if (g) {
       const float z = g[i];
-      y *= z / (1.0f + expf(-z));
+      y *= (sigmoid_gate ? 1.0f : z) / (1.0f + expf(-z));
     }
     Num<T>::st(out + row * vdim + i, y);
   }
@@ -208,7 +212,7 @@ __global__ __launch_bounds__(DS_THREADS) void head_norm_gate_kernel(T* __restric
 extern "C" int ga_decay_scan(void* out, const void* q, const void* k, const void* v, int64_t stride, const void* decay,
                              const void* head_decay, const void* cos_t, const void* sin_t, int rot_dims, float q_scale,
                              float k_scale, void* state, const void* slots, const void* cu, const void* q_start, int entries,
-                             int heads, int dim, int vdim, hipStream_t stream) {
+                             int heads, int dim, int vdim, int silu_inputs, hipStream_t stream) {
   if (entries <= 0) return 0;
   if (heads <= 0 || dim <= 0 || vdim <= 0 || dim > 16 * DS_SLICES) return -1;
   if (heads > 65535 || (vdim + DS_COLS - 1) / DS_COLS > 65535) return -2;
@@ -219,7 +223,7 @@ extern "C" int ga_decay_scan(void* out, const void* q, const void* k, const void
 #define GO(R, T) hipLaunchKernelGGL((decay_scan_kernel<R, T>), grid, block, 0, stream, (float*)out, (const float*)q, (const float*)k, \
                                  (const float*)v, stride, (const float*)decay, (const float*)head_decay, (const float*)cos_t,  \
                                  (const float*)sin_t, rot_dims, q_scale, k_scale, (float*)state, (const int64_t*)slots,       \
-                                 (const int32_t*)cu, (const int32_t*)q_start, heads, dim, vdim)
+                                 (const int32_t*)cu, (const int32_t*)q_start, heads, dim, vdim, silu_inputs)
   if (rows <= 1) GO(1, 16);
   else if (rows <= 2) GO(2, 16);
   else if (rows <= 3) GO(3, 16);
@@ -244,7 +248,8 @@ extern "C" int ga_gla_decay(void* decay, const void* low, int64_t low_stride, co
 }
 
 extern "C" int ga_head_norm_gate(void* out, const void* x, const void* weight, const void* gate, int64_t gate_stride,
-                                 int64_t tokens, int heads, int vdim, float eps, int out_bf16, hipStream_t stream) {
+                                 int64_t tokens, int heads, int vdim, float eps, int out_bf16, int sigmoid_gate,
+                                 int weight_per_head, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (vdim <= 0 || heads <= 0) return -1;
   const int64_t rows = tokens * heads;
@@ -252,9 +257,11 @@ extern "C" int ga_head_norm_gate(void* out, const void* x, const void* weight, c
   dim3 grid((unsigned)((rows + per - 1) / per)), block(DS_THREADS);
   if (out_bf16)
     hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const float*)x,
-                       (const float*)weight, (const float*)gate, gate_stride, rows, heads, vdim, eps);
+                       (const float*)weight, (const float*)gate, gate_stride, rows, heads, vdim, eps, sigmoid_gate,
+                       weight_per_head);
   else
     hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)x,
-                       (const float*)weight, (const float*)gate, gate_stride, rows, heads, vdim, eps);
+                       (const float*)weight, (const float*)gate, gate_stride, rows, heads, vdim, eps, sigmoid_gate,
+                       weight_per_head);
   return GA_CHECK_LAUNCH();
 }

@@ -105,9 +105,9 @@ int ga_embedding_sinusoid_norm(void* out, const void* table, const void* ids, co
 // slots int64 [entries], token_entry int32 [tokens], cu int32 [entries + 1], q_start int32 [entries]
 int ga_short_conv_apply(void* out, const void* x, const void* w, const void* state, const void* slots,
                         const void* token_entry, const void* cu, const void* q_start, int tokens, int width, int taps,
-                        int add_input, int out_bf16, hipStream_t stream);
+                        int add_input, int out_bf16, int64_t x_stride, const void* bias, hipStream_t stream);
 int ga_short_conv_update(void* state, const void* x, const void* slots, const void* cu, const void* q_start, int entries,
-                         int width, int taps, hipStream_t stream);
+                         int width, int taps, int64_t x_stride, hipStream_t stream);
 
 // ---- gated_recurrence.hip: the HGRN2 recurrence.  proj float [tokens, 2 heads dim + heads vdim] (row stride given) holds
 // (q before its SiLU | forget-gate logits | v); state float [slots, heads, dim, vdim]; out float [tokens, heads, vdim]
@@ -192,7 +192,7 @@ int ga_conv_rope_kv(void* q_out, const void* proj, const void* w, void* state, c
                     const void* cu, const void* q_start, const void* positions, const void* cos_t, const void* sin_t,
                     const void* slot_mapping, void* k_pages, void* v_pages, int tokens, int entries, int nh, int nkv, int hd,
                     int vd, int padded, int rotary_dim, int taps, int page_size, int write_kv, int update_state, int is_bf16,
-                    int proj_bf16, hipStream_t stream);
+                    int proj_bf16, void* row_scale, const void* gain, float norm_eps, hipStream_t stream);
 
 // ---- output_norm.hip: residual[t] += scale * gain * y[t] / sqrt(mean(y[t]^2) + eps) (a norm on a sublayer's output, a
 // factor per channel behind it; gain and scale float [hidden], scale may be null); with `next` also next[t] = next_gain *
@@ -209,6 +209,11 @@ int ga_output_norm_add(void* residual, const void* y, const void* gain, const vo
 // width], column c weighted by dense[t, c / ff] (columns behind experts * ff by 1)
 int ga_route_topk(void* ids, void* weights, void* dense, const void* scores, int tokens, int experts, int top,
                   hipStream_t stream);
+// the same outputs from sigmoid scores: choice by s + correction inside the `keep` best of `groups` groups (a group's score:
+// its group_top largest choice scores added), weights s (/ (their sum + floor) where normalise) * scale
+int ga_route_sigmoid_groups(void* ids, void* weights, void* dense, const void* logits, const void* correction, int tokens,
+                            int experts, int top, int groups, int keep, int group_top, int normalise, float floor, float scale,
+                            hipStream_t stream);
 int ga_weighted_silu_mul(void* out, const void* gate_up, const void* dense, int tokens, int width, int experts, int ff,
                          int is_bf16, hipStream_t stream);
 // router scores: scores float [tokens, experts] = w . x + b, 32-bit sums, x in the compute dtype or float
@@ -227,6 +232,8 @@ int ga_combine_pairs(void* out, const void* y, const void* shared, const void* w
 
 // ---- activation.hip: out[i] = max(x[i], 0)^2 over `total` elements (out may be x)
 int ga_relu_square(void* out, const void* x, int64_t total, int is_bf16, hipStream_t stream);
+// out[i] = sa * a[i] + sb * b[i] in 32-bit (two sublayers' results side by side); out may be a or b
+int ga_scaled_sum(void* out, const void* a, const void* b, float sa, float sb, int64_t total, int is_bf16, hipStream_t stream);
 
 // ---- decay_scan.hip: linear attention with a decay as a recurrence, S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per
 // head.  q, k, v: 32-bit rows with a common stride; a from `decay` float [tokens, heads dim] or from `head_decay` float
@@ -236,14 +243,14 @@ int ga_relu_square(void* out, const void* x, int64_t total, int is_bf16, hipStre
 int ga_decay_scan(void* out, const void* q, const void* k, const void* v, int64_t stride, const void* decay,
                   const void* head_decay, const void* cos_t, const void* sin_t, int rot_dims, float q_scale, float k_scale,
                   void* state, const void* slots, const void* cu, const void* q_start, int entries, int heads, int dim,
-                  int vdim, hipStream_t stream);
+                  int vdim, int silu_inputs, hipStream_t stream);
 // decay float [tokens, channels] = sigmoid(a2 low + bias)^(1 / tau); low: 32-bit rows of `rank` numbers with a stride; a2t:
 // a2 transposed, float [rank, channels]
 int ga_gla_decay(void* decay, const void* low, int64_t low_stride, const void* a2t, const void* bias, int tokens,
                  int channels, int rank, float tau, hipStream_t stream);
 // out [tokens, heads, vdim] = x / rms(x over vdim) (* weight [vdim], or null) (* silu(gate), 32-bit rows with a stride, or null)
 int ga_head_norm_gate(void* out, const void* x, const void* weight, const void* gate, int64_t gate_stride, int64_t tokens,
-                      int heads, int vdim, float eps, int out_bf16, hipStream_t stream);
+                      int heads, int vdim, float eps, int out_bf16, int sigmoid_gate, int weight_per_head, hipStream_t stream);
 
 // ---- pooled_attention.hip: attention over a window of tokens and the means of the blocks before it, sigmoid weights.
 // prepare: q and k of a 32-bit projection [q heads | k heads | v heads ...] turned by position (pairs 2i, 2i + 1), divided by
@@ -277,6 +284,28 @@ int ga_pwa_attend_mfma(void* out, void* partial, const void* q, const void* k_ro
 int ga_gated_residual_add(void* residual, const void* z, int64_t z_stride, const void* y1, const void* y2, int tokens, int hidden,
                           int y_bf16,
                           const void* next_gain, float next_eps, void* next, int next_bf16, hipStream_t stream);
+
+// ---- hyper_connection.hip: the residual stream as S streams side by side, X float [tokens, S, width].  open: every stream
+// = x; read: rows = gain * u / rms(u), u = sum_s in[s] X_s; write: X_j <- sum_s mix[s, j] X_s + out[j] * y for all j at once (y
+// in the compute dtype, or float partial sums [parts, tokens, width]) and, where next_in / next_gain / rows are given, the
+// read of the new streams; sum_rows: the streams' sum at the listed rows (rows null: at every row)
+int ga_hc_max_streams();
+int ga_hc_open(void* X, const void* x, int tokens, int width, int streams, hipStream_t stream);
+int ga_hc_read(void* rows, const void* X, const void* in_w, const void* gain, float eps, int tokens, int width, int streams,
+               int rows_bf16, hipStream_t stream);
+int ga_hc_write(void* X, const void* mix, const void* out_w, const void* y, int y_bf16, int parts, int64_t part_stride,
+                const void* next_in, const void* next_gain, float next_eps, void* rows, int rows_bf16, int tokens, int width,
+                int streams, hipStream_t stream);
+int ga_hc_sum_rows(void* out, const void* X, const void* rows, int n_rows, int width, int streams, hipStream_t stream);
+
+// ---- rglru.hip: the real-gated linear recurrent unit.  gates: a = exp(-rate * sigmoid(Ra u + ra) * softplus(lam)), b =
+// sqrt(1 - a^2) * sigmoid(Ri u + ri) * u, the matrices block-diagonal and handed over transposed [block][in][out]; all float
+// [tokens, channels].  scan: S_t = a_t S_(t-1) + b_t per channel over float state [slots, channels] (zeros where an entry's
+// q_start is 0), out = S * gelu_tanh(y), y float rows with a stride
+int ga_rglru_gates(void* a_out, void* b_out, const void* u, const void* ra_t, const void* ra_b, const void* ri_t,
+                   const void* ri_b, const void* lam, int tokens, int channels, int blocks, float rate, hipStream_t stream);
+int ga_rglru_scan(void* out, const void* a, const void* b, const void* y, int64_t y_stride, void* state, const void* slots,
+                  const void* cu, const void* q_start, int entries, int channels, int out_bf16, hipStream_t stream);
 
 // ---- random_fill.hip: out[i] = mean + std * normal(key, i) for n elements, float or bfloat16: the counter-based
 // generator of random_normal.h, which gives the host library (host/random_fill_host.cpp) the same bits

@@ -69,6 +69,106 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_topk_kernel(const float* 
   }
 }
 
+// Routing by sigmoid scores with a correction and groups of experts (one wavefront per token):
+//   s = sigmoid(z);  c = s + correction (the choice score; without a correction c = s)
+//   the experts fall into `groups` equal groups of neighbours; a group's score is the sum of its `group_top` largest c; only
+//   the experts of the `keep` best groups can be chosen (groups == 1: all of them)
+//   the `top` experts with the largest c among those are chosen (the lowest index among equals)
+//   weights: the chosen experts' s, divided by their sum + floor where `normalise`, times `scale`
+// Written as route_topk_kernel writes them: ids and weights [T, top], and a row of weights over all experts.
+#define ROUTE_GROUP_TOP_MAX 4
+__global__ __launch_bounds__(ROUTE_THREADS) void route_sigmoid_groups_kernel(
+    const float* __restrict__ logits, const float* __restrict__ correction, int32_t* __restrict__ ids,
+    float* __restrict__ weights, float* __restrict__ dense, int experts, int top, int groups, int keep, int group_top,
+    int normalise, float floor, float scale) {
+  constexpr int PER = ROUTE_MAX_EXPERTS / ROUTE_THREADS;
+  __shared__ float choice[ROUTE_MAX_EXPERTS], plain[ROUTE_MAX_EXPERTS], group_score[ROUTE_MAX_EXPERTS];
+  __shared__ int32_t kept[ROUTE_MAX_EXPERTS], chosen_i[ROUTE_MAX_EXPERTS];
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x;
+  float c[PER];
+  bool taken[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int e = lane + j * ROUTE_THREADS;
+    float z = e < experts ? logits[t * experts + e] : 0.f;
+    float s = 1.0f / (1.0f + expf(-z));
+    c[j] = e < experts ? s + (correction ? correction[e] : 0.f) : -INFINITY;
+    // what is no number (the rows that pad a recorded step may hold anything) counts as the smallest
+    if (!(c[j] == c[j])) { c[j] = -INFINITY; s = 0.f; }
+    taken[j] = e >= experts;
+    if (e < experts) { choice[e] = c[j]; plain[e] = s; }
+  }
+  __syncthreads();
+  if (groups > 1) {
+    const int n = experts / groups;
+    for (int g = lane; g < groups; g += ROUTE_THREADS) {
+      float best[ROUTE_GROUP_TOP_MAX];
+#pragma unroll
+      for (int k = 0; k < ROUTE_GROUP_TOP_MAX; ++k) best[k] = -INFINITY;
+      for (int i = 0; i < n; ++i) {
+        float v = choice[g * n + i];
+#pragma unroll
+        for (int k = 0; k < ROUTE_GROUP_TOP_MAX; ++k)
+          if (k < group_top && v > best[k]) { const float o = best[k]; best[k] = v; v = o; }
+      }
+      float sum = 0.f;
+#pragma unroll
+      for (int k = 0; k < ROUTE_GROUP_TOP_MAX; ++k)
+        if (k < group_top && k < n) sum += best[k];
+      group_score[g] = sum;
+      kept[g] = 0;
+    }
+    __syncthreads();
+    if (lane == 0) {
+      for (int k = 0; k < keep; ++k) {
+        int at = -1;
+        float best = -INFINITY;
+        for (int g = 0; g < groups; ++g)
+          if (!kept[g] && (at < 0 || group_score[g] > best)) { best = group_score[g]; at = g; }
+        if (at >= 0) kept[at] = 1;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = lane + j * ROUTE_THREADS;
+      if (e < experts && !kept[e / n]) { taken[j] = true; c[j] = -INFINITY; }
+    }
+  }
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = lane + j * ROUTE_THREADS;
+      if (!taken[j] && (at == 0x7fffffff || c[j] > best)) { best = c[j]; at = e; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, WAVE);
+      const int oa = __shfl_xor(at, o, WAVE);
+      if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if (lane + j * ROUTE_THREADS == at) taken[j] = true;
+    if (lane == 0) chosen_i[k] = at < experts ? at : 0;       // top <= the experts that can be chosen: one is always left
+  }
+  __syncthreads();
+  float total = 0.f;
+  for (int k = 0; k < top; ++k) total += plain[chosen_i[k]];             // in the order of the choice
+  const float factor = normalise ? scale / (total + floor) : scale;
+  for (int e = lane; e < experts; e += ROUTE_THREADS) dense[t * experts + e] = 0.f;
+  __syncthreads();
+  for (int k = lane; k < top; k += ROUTE_THREADS) {
+    const float w = plain[chosen_i[k]] * factor;
+    ids[t * top + k] = chosen_i[k];
+    weights[t * top + k] = w;
+    dense[t * experts + chosen_i[k]] = w;
+  }
+}
+
 // gate_up [tokens, 2 * width]: for every expert its ff gate columns and then its ff up columns, the experts one after the
 // other, and behind them the shared expert's (shared gates, then shared ups); out [tokens, width]: expert e's columns at
 // [e * ff, (e + 1) * ff), the shared expert's behind.  V elements a thread in 16-byte accesses where the widths allow it.
@@ -232,6 +332,19 @@ extern "C" int ga_route_topk(void* ids, void* weights, void* dense, const void* 
   if (experts <= 0 || experts > ROUTE_MAX_EXPERTS || top <= 0 || top > experts) return -1;
   hipLaunchKernelGGL(route_topk_kernel, dim3(tokens), dim3(ROUTE_THREADS), 0, stream, (const float*)scores, (int32_t*)ids,
                      (float*)weights, (float*)dense, experts, top);
+  return GA_CHECK_LAUNCH();
+}
+
+extern "C" int ga_route_sigmoid_groups(void* ids, void* weights, void* dense, const void* logits, const void* correction,
+                                       int tokens, int experts, int top, int groups, int keep, int group_top, int normalise,
+                                       float floor, float scale, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (experts <= 0 || experts > ROUTE_MAX_EXPERTS || top <= 0 || top > experts) return -1;
+  if (groups < 1 || experts % groups || keep < 1 || keep > groups || top > keep * (experts / groups)) return -2;
+  if (group_top < 1 || group_top > ROUTE_GROUP_TOP_MAX) return -3;
+  hipLaunchKernelGGL(route_sigmoid_groups_kernel, dim3(tokens), dim3(ROUTE_THREADS), 0, stream, (const float*)logits,
+                     (const float*)correction, (int32_t*)ids, (float*)weights, (float*)dense, experts, top, groups, keep,
+                     group_top, normalise, floor, scale);
   return GA_CHECK_LAUNCH();
 }
 

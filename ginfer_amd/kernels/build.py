@@ -26,7 +26,7 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-shared", "-fPIC",
 MODULES = ("embedding", "norm", "rope_kv", "attention_generic", "attention_mfma", "gemm", "gemm_skinny",
            "activation", "sampling", "random_fill", "scalar_norm", "embedding_sinusoid", "short_conv", "gated_recurrence",
            "latent_attention", "output_norm", "routing", "conv_rope_kv", "decay_scan", "pooled_attention",
-           "gated_residual")
+           "gated_residual", "hyper_connection", "rglru")
 # flags of single modules: the random-weights generator must round every operation by itself, as the host's twin does
 MODULE_FLAGS = {"random_fill": ["-ffp-contract=off"], "attention_generic": ["-ffp-contract=off"]}
 # headers beside common.h that a module includes (they enter its digest)

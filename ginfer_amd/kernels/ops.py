@@ -261,7 +261,7 @@ def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, posit
                             head_dim, scale, window=None, out=None, tokens_per_workgroup=0, sinks=None):
     """q: rows of the fused projection ([T, >= nh*hd]; the first nh*hd columns are the queries).
     Token t attends to the keys of request token_entry[t] at positions
-    [max(0, p - window + 1), p], p = positions[t].  Returns [T, nh*hd].  tokens_per_workgroup: how many neighbouring
+    [max(0, p - window + 1), p], p = positions[t] (window may be any value of `mask_parameter`: negative for chunks).  Returns [T, nh*hd].  tokens_per_workgroup: how many neighbouring
     tokens share a workgroup and (where they are of one request) its tiles of keys and values; 1 suits steps of
     single tokens, 0 leaves it to the library (from 32 tokens on: the matrix cores for a request's 8 tokens and more,
     a second kernel for the requests with fewer), -1 says besides that every request has at least 8 tokens in the
@@ -543,6 +543,26 @@ def qkv_rope_skinny(x, w, bias, positions, cos, sin, slot_mapping, k_pages, v_pa
 MFMA_HEAD_DIMS = tuple(range(16, 257, 16))
 
 
+def mask_parameter(window=None, chunk=None):
+    """The attention kernels' one mask parameter: a sliding window of w keys as w, chunks of c positions counted from
+    position 0 as -c, every earlier key as 0."""
+    _need(not (window and chunk), "a window and chunks at once: %r, %r", window, chunk)
+    if chunk:
+        _need(int(chunk) > 0, "chunks of %r positions", chunk)
+        return -int(chunk)
+    _need(not window or int(window) > 0, "a window of %r keys", window)
+    return int(window) if window else 0
+
+
+def first_visible_key(pos, mask):
+    """The first key that a query at position `pos` sees under the mask parameter (csrc/common.h has the kernels' twin)."""
+    if mask > 0:
+        return max(0, pos - mask + 1)
+    if mask < 0:
+        return pos - pos % (-mask)
+    return 0
+
+
 def attention_mfma_supported(dtype, head_dim, page_size):
     return (dtype == torch.bfloat16 and head_dim in MFMA_HEAD_DIMS and page_size >= 8
             and page_size & (page_size - 1) == 0)
@@ -624,7 +644,7 @@ def key_parts(tiles, tile_rows, window, workgroups_per_tile, streams, compute_un
     size 128: 40.8 us whole, 45.6 in parts: the workgroups beyond one round of the chip pay a workgroup's fixed part, some
     8 us, a second time, and the merge and 10 MB of partial results cost what the shorter walks save)."""
     def key_tiles(t):
-        lo = max(0, t[3] - window + 1) if window else 0
+        lo = first_visible_key(t[3], window or 0)
         return (t[3] + t[2] - 1) // 32 + 1 - lo // 32, (lo // 32) * 32
     counts = [key_tiles(t)[0] for t in tiles]
     heaviest = max(counts)
@@ -657,10 +677,10 @@ def key_parts(tiles, tile_rows, window, workgroups_per_tile, streams, compute_un
 def _decode_splits(plan, window, nkv, head_blocks):
     span = 0
     if plan.get("decode_span"):             # a recorded step: the split must fit every context of its bucket
-        span = plan["decode_span"] if not window else min(plan["decode_span"], (window + 62) // 32 * 32)
+        span = plan["decode_span"] if not window else min(plan["decode_span"], (abs(window) + 62) // 32 * 32)
     else:
         for pos in plan["decode_pos"]:
-            lo = max(0, pos - window + 1) if window else 0
+            lo = first_visible_key(pos, window or 0)
             span = max(span, pos + 1 - (lo // 32) * 32)
     per_split = plan["n_decode"] * nkv * head_blocks
     splits = max(1, min(TUNING.decode_target_workgroups // max(per_split, 1), -(-span // TUNING.decode_min_split_keys),
@@ -754,11 +774,13 @@ def _prefill_workgroups(step, tile_rows, group, nkv, head_dim, window):
 
 
 def paged_attention(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale, window=None,
-                    sinks=None):
-    """Attention of every token of the step over its request's pages.  Chooses the kernel: the general
+                    sinks=None, chunk=None):
+    """Attention of every token of the step over its request's pages.  window: the last `window` keys; chunk: the keys of
+    the query's own chunk of `chunk` positions, counted from position 0 (neither: every earlier key).  Chooses the kernel: the general
     one in 32-bit (fixed order of every sum: bit-identical however the work is cut); in bfloat16 the
     matrix-core kernels where they take the shape.  sinks: None, or float32 [num_heads], a score per head that
     enters every denominator of the softmax and has no value."""
+    window = mask_parameter(window, chunk) or None
     if attention_mfma_supported(q.dtype, head_dim, k_pages.shape[2]):
         return paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale,
                                     window, sinks=sinks)
@@ -853,13 +875,16 @@ def embedding_sinusoid_norm(table, ids, positions, freq, gain, eps):
 SHORT_CONV_MAX_TAPS = 16
 
 
-def short_conv(x, weight, state, slots, step, dtype, add_input=True, update=True):
-    """x float32 [T, W] (the residual stream); weight float32 [W, taps]; state float32 [slots, taps - 1, W] (None for one
-    tap); slots int64 [entries].  Returns (x +) the causal convolution in `dtype`, the inputs before the step's tokens
-    taken from the state, and moves the state on by the step's tokens."""
-    _dev(x, weight, state, slots)
-    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "x must be contiguous float32 [T, W]")
+def short_conv(x, weight, state, slots, step, dtype, add_input=True, update=True, bias=None):
+    """x float32 [T, W] (the residual stream, or columns of a wider 32-bit tensor); weight float32 [W, taps]; state float32
+    [slots, taps - 1, W] (None for one tap); slots int64 [entries]; bias float32 [W] or None.  Returns (x +) the causal
+    convolution (+ bias) in `dtype`, the inputs before the step's tokens taken from the state, and moves the state on by the
+    step's tokens."""
+    _dev(x, weight, state, slots, bias)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1, "x must be float32 [T, W] with unit inner stride")
     T, W = x.shape
+    if bias is not None:
+        _f32(bias, (W,), "bias")
     _need(weight.dim() == 2 and weight.shape[0] == W and 1 <= weight.shape[1] <= SHORT_CONV_MAX_TAPS,
           "the convolution's weight must be [%d, taps <= %d], got %s", W, SHORT_CONV_MAX_TAPS, tuple(weight.shape))
     taps = weight.shape[1]
@@ -875,10 +900,10 @@ def short_conv(x, weight, state, slots, step, dtype, add_input=True, update=True
     lib = build.load("short_conv")
     _check(lib.ga_short_conv_apply(_ptr(out), _ptr(x), _ptr(weight), _ptr(state), _ptr(slots), _ptr(step.token_entry),
                                    _ptr(step.cu_tokens), _ptr(step.q_start), _i(T), _i(W), _i(taps), _i(1 if add_input else 0),
-                                   _i(_is_bf16(dtype)), _stream()), "short_conv_apply")
+                                   _i(_is_bf16(dtype)), _i64(x.stride(0)), _ptr(bias), _stream()), "short_conv_apply")
     if update and taps > 1:
         _check(lib.ga_short_conv_update(_ptr(state), _ptr(x), _ptr(slots), _ptr(step.cu_tokens), _ptr(step.q_start), _i(E), _i(W),
-                                        _i(taps), _stream()), "short_conv_update")
+                                        _i(taps), _i64(x.stride(0)), _stream()), "short_conv_update")
     return out
 
 
@@ -1080,6 +1105,31 @@ def route_topk(scores, top):
     return ids, weights, dense
 
 
+def route_sigmoid_groups(logits, top, correction=None, groups=1, keep=1, group_top=2, normalise=True, floor=0.0, scale=1.0):
+    """logits float32 [T, E] -> (ids, weights, dense) as `route_topk` gives them, from sigmoid scores s = sigmoid(logits): the
+    choice goes by s + correction (float32 [E] or None); the experts fall into `groups` equal groups of neighbours, a group's
+    score is the sum of its `group_top` largest choice scores, and only experts of the `keep` best groups can be chosen; the
+    weights are the chosen experts' s, divided by their sum + floor where `normalise`, times scale."""
+    _dev(logits, correction)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "logits must be contiguous float32 [T, E]")
+    T, E = logits.shape
+    _need(1 <= E <= ROUTE_MAX_EXPERTS and 1 <= top <= E, "routing takes 1 to %d experts and 1 <= top <= experts; got %d, top %d",
+          ROUTE_MAX_EXPERTS, E, top)
+    _need(groups >= 1 and E % groups == 0 and 1 <= keep <= groups and top <= keep * (E // groups) and 1 <= group_top <= 4,
+          "%d experts in %d groups of which %d are kept (scored by their %d largest) cannot give %d choices", E, groups, keep,
+          group_top, top)
+    if correction is not None:
+        _f32(correction, (E,), "correction")
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    dense = torch.empty((T, E), dtype=torch.float32, device=logits.device)
+    lib = build.load("routing")
+    _check(lib.ga_route_sigmoid_groups(_ptr(ids), _ptr(weights), _ptr(dense), _ptr(logits), _ptr(correction), _i(T), _i(E), _i(top),
+                                       _i(groups), _i(keep), _i(group_top), _i(1 if normalise else 0), _f(floor), _f(scale),
+                                       _stream()), "route_sigmoid_groups")
+    return ids, weights, dense
+
+
 def router_scores(x, weight, bias):
     """x [T, H] (bfloat16 or float32), weight float32 [E, H], bias float32 [E] or None -> float32 [T, E] = x . weight^T + bias,
     summed in 32-bit, a wavefront per score."""
@@ -1179,11 +1229,24 @@ def relu_square(x):
     return x
 
 
+def scaled_sum(a, b, sa, sb):
+    """sa * a + sb * b in 32-bit, written over a; a and b contiguous and alike (float32 or bfloat16)."""
+    _dev(a, b)
+    _need(a.shape == b.shape and a.dtype == b.dtype and a.is_contiguous() and b.is_contiguous()
+          and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0, "a and b must be contiguous and alike at 16-byte addresses")
+    lib = build.load("activation")
+    _check(lib.ga_scaled_sum(_ptr(a), _ptr(a), _ptr(b), _f(sa), _f(sb), _i64(a.numel()), _i(_is_bf16(a.dtype)), _stream()),
+           "scaled_sum")
+    return a
+
+
 def conv_rope_kv(proj, weight, state, slots, step, cos, sin, slot_mapping, k_pages, v_pages, num_heads, num_kv_heads, head_dim,
-                 value_dim, padded, dtype, write_kv=True, update_state=True):
+                 value_dim, padded, dtype, write_kv=True, update_state=True, qk_gain=None, qk_eps=0.0):
     """Behind a fused q|k|v projection whose channels pass a short causal convolution: proj [T, (nh + nkv) hd + nkv vd] in
     the compute dtype `dtype` or in float32; weight float32 [channels, taps] (None: no convolution); state float32 [slots, taps - 1, channels]
     (None for one tap) and slots int64 [entries]; cos, sin float32 [positions, rotary_dim / 2] (None: no rotation).
+    qk_gain float32 [(nh + nkv) hd] (no convolution then): q and k are divided by the root mean square of the token's WHOLE q
+    (k) projection (eps qk_eps) and multiplied by the gain, before the rotation.
     Returns q [T, nh * padded], heads padded with zeros, and writes k and v (padded alike) into the pages at slot_mapping;
     moves the state on by the step's tokens."""
     _dev(proj, weight, state, slots, cos, sin, slot_mapping, k_pages, v_pages)
@@ -1221,13 +1284,19 @@ def conv_rope_kv(proj, weight, state, slots, step, cos, sin, slot_mapping, k_pag
         page_size = _check_pages(k_pages, v_pages, dtype, num_kv_heads, padded)
     _need(proj.dtype in (dtype, torch.float32), "proj must be %s or float32", dtype)
     q = torch.empty((T, num_heads * padded), dtype=dtype, device=proj.device)
+    row_scale = None
+    if qk_gain is not None:
+        _need(weight is None, "the norm over the whole projection stands in front of no convolution")
+        _f32(qk_gain, ((num_heads + num_kv_heads) * head_dim,), "qk_gain")
+        _need(qk_gain.device == proj.device, "qk_gain lies on another device")
+        row_scale = torch.empty((T, 2), dtype=torch.float32, device=proj.device)
     lib = build.load("conv_rope_kv")
     _check(lib.ga_conv_rope_kv(_ptr(q), _ptr(proj), _ptr(weight), _ptr(state), _ptr(slots), _ptr(step.token_entry),
                                _ptr(step.cu_tokens), _ptr(step.q_start), _ptr(step.positions), _ptr(cos), _ptr(sin),
                                _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), _i(T), _i(E), _i(num_heads), _i(num_kv_heads),
                                _i(head_dim), _i(value_dim), _i(padded), _i(rotary_dim), _i(taps), _i(page_size),
                                _i(1 if write_kv else 0), _i(1 if update_state else 0), _i(_is_bf16(dtype)),
-                               _i(_is_bf16(proj.dtype)), _stream()),
+                               _i(_is_bf16(proj.dtype)), _ptr(row_scale), _ptr(qk_gain), _f(qk_eps), _stream()),
            "conv_rope_kv")
     return q
 
@@ -1272,13 +1341,13 @@ def gla_decay(proj, low_start, a2t, bias, tau):
 
 
 def decay_scan(proj, q_start, k_start, v_start, state, slots, step, heads, dim, vdim, decay=None, head_decay=None, cos=None,
-               sin=None, q_scale=1.0, k_scale=1.0):
+               sin=None, q_scale=1.0, k_scale=1.0, silu_inputs=False):
     """Linear attention with a decay as a recurrence over per-request state: S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T
     q_t per head.  q, k, v are column blocks of the float32 projection `proj` (starting at q_start, k_start, v_start; heads *
     dim, heads * dim, heads * vdim wide).  a: `decay` float32 [T, heads * dim], or `head_decay` float32 [heads].  cos, sin
     float32 [positions, r / 2]: q and k are turned on their first r coordinates (pairs i, i + r / 2) by the tokens' positions,
     then multiplied by q_scale and k_scale.  state float32 [slots, heads, dim, vdim] is advanced in place (zeros where an
-    entry's q_start is 0).  Returns float32 [T, heads, vdim]."""
+    entry's q_start is 0).  silu_inputs: the recurrence reads silu(q), silu(k) and silu(v).  Returns float32 [T, heads, vdim]."""
     _dev(proj, state, slots, decay, head_decay, cos, sin)
     T = proj.shape[0]
     q = _rows_of(proj, q_start, heads * dim, "q")
@@ -1304,14 +1373,15 @@ def decay_scan(proj, q_start, k_start, v_start, state, slots, step, heads, dim, 
     lib = build.load("decay_scan")
     _check(lib.ga_decay_scan(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _i64(proj.stride(0)), _ptr(decay), _ptr(head_decay),
                              _ptr(cos), _ptr(sin), _i(rot), _f(q_scale), _f(k_scale), _ptr(state), _ptr(slots),
-                             _ptr(step.cu_tokens), _ptr(step.q_start), _i(E), _i(heads), _i(dim), _i(vdim), _stream()), "decay_scan")
+                             _ptr(step.cu_tokens), _ptr(step.q_start), _i(E), _i(heads), _i(dim), _i(vdim),
+                             _i(1 if silu_inputs else 0), _stream()), "decay_scan")
     return out
 
 
-def head_norm_gate(x, weight, eps, dtype, proj=None, gate_start=0):
+def head_norm_gate(x, weight, eps, dtype, proj=None, gate_start=0, sigmoid_gate=False):
     """x float32 [T, heads, V] -> [T, heads * V] in `dtype`: every head's row divided by its root mean square, times weight
-    [V] (None: no weight), times silu of the gate, the columns gate_start .. gate_start + heads * V of the float32
-    projection `proj` (None: no gate)."""
+    [V] (None: no weight), times silu of the gate (its sigmoid where sigmoid_gate), the columns gate_start .. gate_start +
+    heads * V of the float32 projection `proj` (None: no gate).  A norm over all heads together is the case heads = 1."""
     _dev(x, weight, proj)
     _need(x.dtype == torch.float32 and x.dim() == 3 and x.is_contiguous(), "x must be contiguous float32 [T, heads, V]")
     T, H, V = x.shape
@@ -1324,7 +1394,8 @@ def head_norm_gate(x, weight, eps, dtype, proj=None, gate_start=0):
     out = torch.empty((T, H * V), dtype=dtype, device=x.device)
     lib = build.load("decay_scan")
     _check(lib.ga_head_norm_gate(_ptr(out), _ptr(x), _ptr(weight), _ptr(gate), _i64(proj.stride(0) if proj is not None else 0),
-                                 _i64(T), _i(H), _i(V), _f(eps), _i(_is_bf16(dtype)), _stream()), "head_norm_gate")
+                                 _i64(T), _i(H), _i(V), _f(eps), _i(_is_bf16(dtype)), _i(1 if sigmoid_gate else 0), _i(0),
+                                 _stream()), "head_norm_gate")
     return out
 
 
@@ -1489,3 +1560,127 @@ def gated_residual_add(residual, z, y1, y2=None, next_gain=None, next_eps=0.0, d
                                      _ptr(next_gain), _f(next_eps), _ptr(nxt), _i(_is_bf16(dtype) if nxt is not None else 0),
                                      _stream()), "gated_residual_add")
     return nxt
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# hyper-connections: the residual stream as several streams side by side
+
+HYPER_MAX_STREAMS = 8
+HYPER_MAX_WIDTH = 15360          # a token's row of 32-bit sums lies in LDS
+
+
+def _streams(X):
+    _need(X.dtype == torch.float32 and X.dim() == 3 and X.is_contiguous(), "the streams must be contiguous float32 [T, S, W]")
+    T, S, W = X.shape
+    _need(1 <= S <= HYPER_MAX_STREAMS and 1 <= W <= HYPER_MAX_WIDTH, "1 to %d streams of up to %d channels, got %d of %d",
+          HYPER_MAX_STREAMS, HYPER_MAX_WIDTH, S, W)
+    return T, S, W
+
+
+def hyper_open(x, streams):
+    """x float32 [T, W] -> float32 [T, streams, W]: every stream a copy of x."""
+    _dev(x)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "x must be contiguous float32 [T, W]")
+    X = torch.empty((x.shape[0], int(streams), x.shape[1]), dtype=torch.float32, device=x.device)
+    T, S, W = _streams(X)
+    _check(build.load("hyper_connection").ga_hc_open(_ptr(X), _ptr(x), _i(T), _i(W), _i(S), _stream()), "hc_open")
+    return X
+
+
+def hyper_read(X, in_weights, gain, eps, dtype):
+    """rows [T, W] in `dtype` = gain * u / sqrt(mean(u^2) + eps), u = sum_s in_weights[s] X[:, s]."""
+    _dev(X, in_weights, gain)
+    T, S, W = _streams(X)
+    _f32(in_weights, (S,), "in_weights")
+    _f32(gain, (W,), "gain")
+    rows = torch.empty((T, W), dtype=dtype, device=X.device)
+    _check(build.load("hyper_connection").ga_hc_read(_ptr(rows), _ptr(X), _ptr(in_weights), _ptr(gain), _f(eps), _i(T), _i(W), _i(S),
+                                                     _i(_is_bf16(dtype)), _stream()), "hc_read")
+    return rows
+
+
+def hyper_write(X, mix, out_weights, y, next_in=None, next_gain=None, next_eps=0.0, dtype=None):
+    """X[:, j] <- sum_s mix[s, j] X[:, s] + out_weights[j] * y for all j at once, in place.  y [T, W] in float32 or bfloat16, or
+    float32 [parts, T, W] (partial sums, added in order).  With next_in (float32 [S]) and next_gain (float32 [W]) the rows that
+    the sublayer which runs next reads of the new streams (`hyper_read`) come back in `dtype`; else None."""
+    _dev(X, mix, out_weights, y, next_in, next_gain)
+    T, S, W = _streams(X)
+    _f32(mix, (S, S), "mix")
+    _f32(out_weights, (S,), "out_weights")
+    parts, part_stride = 1, 0
+    if y.dim() == 3:
+        _need(y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape[1:]) == (T, W), "partial sums must be contiguous float32 [parts, %d, %d]", T, W)
+        parts, part_stride = y.shape[0], T * W
+    else:
+        _need(tuple(y.shape) == (T, W) and y.is_contiguous() and y.dtype in (torch.float32, torch.bfloat16),
+              "y must be contiguous float32 or bfloat16 [%d, %d], got %s %s", T, W, y.dtype, tuple(y.shape))
+    rows = None
+    _need((next_in is None) == (next_gain is None), "the next sublayer's weights and its norm's gain come together")
+    if next_in is not None:
+        _f32(next_in, (S,), "next_in")
+        _f32(next_gain, (W,), "next_gain")
+        rows = torch.empty((T, W), dtype=dtype, device=X.device)
+    _check(build.load("hyper_connection").ga_hc_write(
+        _ptr(X), _ptr(mix), _ptr(out_weights), _ptr(y), _i(_is_bf16(y.dtype)), _i(parts), _i64(part_stride), _ptr(next_in),
+        _ptr(next_gain), _f(next_eps), _ptr(rows), _i(_is_bf16(dtype) if rows is not None else 0), _i(T), _i(W), _i(S), _stream()),
+        "hc_write")
+    return rows
+
+
+def hyper_sum(X, rows=None):
+    """float32 [R, W]: the sum of the streams at the rows `rows` (int32 [R]; None: at every row)."""
+    _dev(X, rows)
+    T, S, W = _streams(X)
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be contiguous int32 [R]")
+    R = T if rows is None else rows.shape[0]
+    out = torch.empty((R, W), dtype=torch.float32, device=X.device)
+    _check(build.load("hyper_connection").ga_hc_sum_rows(_ptr(out), _ptr(X), _ptr(rows), _i(R), _i(W), _i(S), _stream()), "hc_sum_rows")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the real-gated linear recurrent unit
+
+RGLRU_MAX_BLOCK = 1920           # eight tokens' channels of a block lie in LDS
+
+
+def rglru_gates(u, ra_t, ra_bias, ri_t, ri_bias, lam, blocks, rate):
+    """u float32 [T, C] -> (a, b) float32 [T, C]: per block of C / blocks channels r = sigmoid(Ra u + ra), i = sigmoid(Ri u +
+    ri); a = exp(-rate * r * softplus(lam)); b = sqrt(1 - a^2) * i * u.  ra_t, ri_t: the blocks' square matrices transposed,
+    float32 [blocks, in, out]; the biases and lam float32 [C]."""
+    _dev(u, ra_t, ra_bias, ri_t, ri_bias, lam)
+    _need(u.dtype == torch.float32 and u.dim() == 2 and u.is_contiguous(), "u must be contiguous float32 [T, C]")
+    T, C = u.shape
+    _need(blocks >= 1 and C % blocks == 0 and C // blocks <= RGLRU_MAX_BLOCK, "%d channels in %d blocks (a block may hold up to %d)",
+          C, blocks, RGLRU_MAX_BLOCK)
+    bw = C // blocks
+    for name, t in (("ra_t", ra_t), ("ri_t", ri_t)):
+        _f32(t, (blocks, bw, bw), name)
+    for name, t in (("ra_bias", ra_bias), ("ri_bias", ri_bias), ("lam", lam)):
+        _f32(t, (C,), name)
+    a = torch.empty((T, C), dtype=torch.float32, device=u.device)
+    b = torch.empty((T, C), dtype=torch.float32, device=u.device)
+    _check(build.load("rglru").ga_rglru_gates(_ptr(a), _ptr(b), _ptr(u), _ptr(ra_t), _ptr(ra_bias), _ptr(ri_t), _ptr(ri_bias), _ptr(lam),
+                                              _i(T), _i(C), _i(blocks), _f(rate), _stream()), "rglru_gates")
+    return a, b
+
+
+def rglru_scan(a, b, y, state, slots, step, dtype):
+    """S_t = a_t S_(t-1) + b_t per channel over the step's entries, from the state float32 [slots, C] (zeros where an entry's
+    q_start is 0), which moves on in place; returns S * gelu_tanh(y) in `dtype`, [T, C].  a, b float32 [T, C]; y float32 [T, C]
+    with unit inner stride (columns of a projection, before their activation)."""
+    _dev(a, b, y, state, slots)
+    _need(a.dtype == torch.float32 and a.dim() == 2 and a.is_contiguous(), "a must be contiguous float32 [T, C]")
+    T, C = a.shape
+    _f32(b, (T, C), "b")
+    _need(y.dtype == torch.float32 and tuple(y.shape) == (T, C) and y.stride(1) == 1, "y must be float32 [%d, %d] with unit inner stride", T, C)
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == C and state.is_contiguous(),
+          "state must be contiguous float32 [slots, %d]", C)
+    E = _step_entries(step, slots)
+    _need(E <= 65535, "too many entries for one launch: %d", E)
+    out = torch.empty((T, C), dtype=dtype, device=a.device)
+    _check(build.load("rglru").ga_rglru_scan(_ptr(out), _ptr(a), _ptr(b), _ptr(y), _i64(y.stride(0)), _ptr(state), _ptr(slots),
+                                             _ptr(step.cu_tokens), _ptr(step.q_start), _i(E), _i(C), _i(_is_bf16(dtype)), _stream()),
+           "rglru_scan")
+    return out

@@ -245,3 +245,53 @@ class ParallelGatedBlock(Arrangement):
             results.append(self.feed_forward.forward(n))
         rows = self.gate.add(residual, z, [whole(r).to(n.dtype) if r.dim() == 3 else r for r in results], then=into_norm)
         return NormedRows(rows) if into_norm is not None else None
+
+
+@register_arrangement("hyper_prenorm")
+class HyperPreNormBlock(Arrangement):
+    """A pre-norm block around several residual streams X (float32 [T, S, W]; the model's `stream` part makes them): every
+    sublayer reads the norm of a weighted sum of the streams and writes its result back into all of them through its
+    connection (a part of the `connection` family: `read(X, norm)`, `write(X, y, then)`), first the mixer, then the
+    feed-forward; a layer may have no feed-forward (then neither its norm nor its connection).  The launch that writes a
+    sublayer's result also makes the rows that the next sublayer reads: the feed-forward's inside the block, and the next
+    block's mixer's where the model hands that block's first connection and norm over (`into_norm`; the next block then
+    gets `NormedRows` in place of a delta).  The streams are updated in place; nothing is left pending."""
+
+    roles = {"mixer": "mixer", "mixer_norm": "norm", "mixer_link": "connection", "feed_forward": "feed_forward",
+             "feed_forward_norm": "norm", "feed_forward_link": "connection"}
+    optional_roles = ("feed_forward", "feed_forward_norm", "feed_forward_link")
+
+    folds_output = True              # forward() takes `into_norm`
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.feed_forward = self._parts.get("feed_forward")
+        self.feed_forward_norm = self._parts.get("feed_forward_norm")
+        self.feed_forward_link = self._parts.get("feed_forward_link")
+        present = [p is not None for p in (self.feed_forward, self.feed_forward_norm, self.feed_forward_link)]
+        if any(present) != all(present):
+            raise ValueError("a block names its feed-forward, that feed-forward's norm and its connection together, or none of them")
+        for norm in (self.mixer_norm, self.feed_forward_norm):
+            if norm is not None and not SandwichBlock._plain_gain(norm):
+                raise ValueError("the norms of this block are plain gains over the root mean square: %s is not" % type(norm).__name__)
+
+    def takes_folded_input(self):
+        """(connection, norm) of the block's first sublayer: the block before can make its rows."""
+        return (self.mixer_link, self.mixer_norm)
+
+    def forward(self, residual, delta, step, cache, into_norm=None):
+        if residual.dim() != 3:
+            raise ValueError("this block runs around several streams [T, S, W]; the model needs a `stream` part")
+        if isinstance(delta, NormedRows):
+            n = delta.rows
+        else:
+            if delta is not None:
+                raise ValueError("a block around several streams cannot take another block's pending output")
+            n = self.mixer_link.read(residual, self.mixer_norm)
+        m = self.mixer.forward(n, step, cache)
+        if self.feed_forward is None:
+            rows = self.mixer_link.write(residual, m, then=into_norm)
+            return NormedRows(rows) if into_norm is not None else None
+        n = self.mixer_link.write(residual, m, then=(self.feed_forward_link, self.feed_forward_norm))
+        rows = self.feed_forward_link.write(residual, self.feed_forward.forward(n), then=into_norm)
+        return NormedRows(rows) if into_norm is not None else None

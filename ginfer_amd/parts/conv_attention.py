@@ -1,4 +1,5 @@
-"""Attention whose projections pass a short convolution over time, with values of their own width and a sink."""
+"""Attention with values of their own width: optionally a short convolution over time behind the projections, a norm over
+the whole projection of q and of k, biases, a sink (one score for all heads, or a learned one per head), a window or chunks."""
 import torch
 
 from ..kernels import ops
@@ -27,8 +28,15 @@ class ConvAttention(Part):
 
     capturable = True
 
+    LEARNED = "learned"
+
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, value_dim, scale, dtype, device, taps=None,
-                 position=None, sink=None, window=None, names=None):
+                 position=None, sink=None, window=None, names=None, chunk=None, bias=False, qk_norm_eps=None):
+        """Beyond the class's text: sink = ConvAttention.LEARNED reads one score per head from the tensor `sink`; chunk: a
+        token sees the earlier tokens of its own chunk of `chunk` positions, counted from position 0 (in place of a
+        window); bias: q, k, v and o have biases (`<name>.b`); qk_norm_eps: q and k are divided by the root mean square of
+        the token's whole q (k) projection, all heads at once, and multiplied by the gains `q.norm`, `k.norm`, before the
+        rotation (no convolution then)."""
         if num_heads % num_kv_heads:
             raise ValueError("num_heads %d is not a multiple of num_kv_heads %d" % (num_heads, num_kv_heads))
         self.hidden_size, self.nh, self.nkv = int(hidden_size), int(num_heads), int(num_kv_heads)
@@ -45,16 +53,25 @@ class ConvAttention(Part):
         if position is not None and position.rotary_dim > self.hd:
             raise ValueError("the rotation covers %d coordinates of a head of %d" % (position.rotary_dim, self.hd))
         self.scale = float(scale)
-        self.sink = None if sink is None else float(sink)
+        self.learned_sink = sink == self.LEARNED
+        self.sink = None if sink is None or self.learned_sink else float(sink)
         self.window = int(window) if window else None
-        self.names = dict(q="q", k="k", v="v", o="o", conv="conv")
+        self.chunk = int(chunk) if chunk else None
+        if self.window and self.chunk:
+            raise ValueError("a window and chunks at once: %r, %r" % (window, chunk))
+        self.bias = bool(bias)
+        self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
+        if self.qk_norm_eps is not None and taps:
+            raise ValueError("the norm over the whole projection stands in front of no convolution")
+        self.names = dict(q="q", k="k", v="v", o="o", conv="conv", sink="sink", bias="b", norm="norm")
         self.names.update(names or {})
         self.dtype, self.device = dtype, device
         self.width = (self.nh + self.nkv) * self.hd + self.nkv * self.vd        # the projection's channels
-        self.w_qkv = self.w_conv = self.w_o = self.sinks = None
+        self.w_qkv = self.w_conv = self.w_o = self.sinks = self.b_qkv = self.b_o = self.qk_gain = None
 
     def cache_spec(self):
-        """[the convolution's state (or None), the pages of keys and values]."""
+        """[the convolution's state (or None), the pages of keys and values].  Chunks keep every page: the keys before a
+        token's chunk are never read again, but nothing gives them back before the request ends."""
         state = StateSpec((self.taps - 1, self.width), torch.float32) if self.taps > 1 else None
         return [state, KVCacheSpec(self.nkv, self.padded, self.window)]
 
@@ -66,6 +83,15 @@ class ConvAttention(Part):
         if self.has_conv:
             for r in ("q", "k", "v"):
                 specs[n[r] + "." + n["conv"]] = WeightSpec((rows[r], self.taps), std=0.5, keep_32bit=True)
+        if self.bias:
+            for r in ("q", "k", "v"):
+                specs[n[r] + "." + n["bias"]] = WeightSpec((rows[r],), std=0.1)
+            specs[n["o"] + "." + n["bias"]] = WeightSpec((H,), std=0.1)
+        if self.learned_sink:
+            specs[n["sink"]] = WeightSpec((self.nh,), std=1.0, keep_32bit=True)
+        if self.qk_norm_eps is not None:
+            for r in ("q", "k"):
+                specs[n[r] + "." + n["norm"]] = WeightSpec((rows[r],), init="one_plus_normal", keep_32bit=True)
         return specs
 
     def _padded_rows(self, t, heads, width):
@@ -85,6 +111,13 @@ class ConvAttention(Part):
         self.w_o = self._padded_rows(w_o.t().contiguous(), self.nh, self.vd).t().contiguous()
         dev = self.w_qkv.device
         self.sinks = None if self.sink is None else torch.full((self.nh,), self.sink, dtype=torch.float32, device=dev)
+        if self.learned_sink:
+            self.sinks = t[n["sink"]].float().contiguous()
+        if self.bias:
+            self.b_qkv = torch.cat([t[n[r] + "." + n["bias"]] for r in ("q", "k", "v")], dim=0).contiguous()
+            self.b_o = t[n["o"] + "." + n["bias"]].contiguous()
+        if self.qk_norm_eps is not None:
+            self.qk_gain = torch.cat([t[n[r] + "." + n["norm"]].float() for r in ("q", "k")], dim=0).contiguous()
 
     def kernel_modules(self):
         mods = ["conv_rope_kv", "attention_generic", "gemm"]
@@ -98,10 +131,12 @@ class ConvAttention(Part):
         state, kv = cache
         cos, sin = self.position.tables() if self.position is not None else (None, None)
         # the projection's rows stay 32-bit until they are convolved and rotated: what is cached is rounded once
-        q = ops.conv_rope_kv(linear(x, self.w_qkv, None, out_dtype=torch.float32), self.w_conv, None if state is None else state.state,
+        q = ops.conv_rope_kv(linear(x, self.w_qkv, self.b_qkv, out_dtype=torch.float32), self.w_conv,
+                             None if state is None else state.state,
                              None if state is None else state.slots, step, cos, sin, kv.slot_mapping, kv.k_pages, kv.v_pages,
                              self.nh, self.nkv, self.hd, self.vd, self.padded, self.dtype, write_kv=kv.owner,
-                             update_state=state is not None and state.owner)
+                             update_state=state is not None and state.owner, qk_gain=self.qk_gain,
+                             qk_eps=self.qk_norm_eps or 0.0)
         a = ops.paged_attention(q, kv.k_pages, kv.v_pages, kv.block_table, step, self.nh, self.nkv, self.padded,
-                                self.scale, self.window, sinks=self.sinks)
-        return linear(a, self.w_o, None, parts_ok=True)
+                                self.scale, self.window, sinks=self.sinks, chunk=self.chunk)
+        return linear(a, self.w_o, self.b_o, parts_ok=self.b_o is None)

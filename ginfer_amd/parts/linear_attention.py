@@ -136,3 +136,37 @@ class Retention(_DecayedLinearAttention):
                            head_decay=self.head_decay, cos=cos, sin=sin, k_scale=self.dk ** -0.5)
         o = ops.head_norm_gate(o, None, self.eps, self.dtype, proj=proj, gate_start=self._g0)
         return linear(o, self.w_o)
+
+
+@register_mixer("lightning")
+class LightningAttention(_DecayedLinearAttention):
+    """q = silu(Wq x), k = silu(Wk x), v = silu(Wv x); head h decays by the constant decay[h] and nothing else scales; the
+    heads' outputs side by side are divided by the root mean square over ALL of them at once, times a weight per channel,
+    times sigmoid(Wg x); then Wo.  Tensors: q, k, v, g, o, norm."""
+
+    def __init__(self, hidden_size, num_heads, key_dim, value_dim, decay, eps, dtype, device):
+        super().__init__(hidden_size, num_heads, key_dim, value_dim, eps, dtype, device)
+        self.decay = [float(d) for d in decay]
+        if len(self.decay) != self.nh:
+            raise ValueError("%d decays for %d heads" % (len(self.decay), self.nh))
+        self.head_decay = self.norm_weight = None
+
+    def weight_specs(self):
+        specs = self._projection_specs()
+        specs["norm"] = WeightSpec((self.nh * self.dv,), init="one_plus_normal", keep_32bit=True)
+        return specs
+
+    def bind_weights(self, t):
+        self.w_in = torch.cat([t["q"], t["k"], t["v"], t["g"]], dim=0).contiguous()
+        self.w_o = t["o"]
+        self.norm_weight = t["norm"].float().contiguous()
+        self.head_decay = torch.tensor(self.decay, dtype=torch.float32, device=self.w_in.device)
+
+    def forward(self, x, step, cache):
+        proj = self._project(x)
+        o = ops.decay_scan(proj, 0, self._k0, self._v0, cache.state, cache.slots, step, self.nh, self.dk, self.dv,
+                           head_decay=self.head_decay, silu_inputs=True)
+        # the norm runs over the heads together: one "head" as wide as all of them
+        o = ops.head_norm_gate(o.view(o.shape[0], 1, self.nh * self.dv), self.norm_weight, self.eps, self.dtype, proj=proj,
+                               gate_start=self._g0, sigmoid_gate=True)
+        return linear(o, self.w_o, parts_ok=True)

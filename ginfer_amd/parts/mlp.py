@@ -128,7 +128,26 @@ class RoutedGLU(Part):
 
     capturable = True                # the steps that the runner records are short enough for the first way
 
-    def __init__(self, hidden_size, num_experts, top_k, expert_size, dtype, device, shared_size=None, router_bias=True):
+    def __init__(self, hidden_size, num_experts, top_k, expert_size, dtype, device, shared_size=None, router_bias=True,
+                 scoring="softmax_chosen", correction=False, groups=1, keep_groups=1, group_top=2, weight_scale=1.0,
+                 weight_floor=0.0):
+        """scoring "softmax_chosen": as the class's text.  scoring "sigmoid": scores s = sigmoid(z); the choice goes by s +
+        `correction` (a tensor of that name, where correction is set) among the experts of the `keep_groups` best of `groups`
+        equal groups of neighbouring experts (a group's score: the sum of its `group_top` largest choice scores); the weights
+        are the chosen experts' s divided by their sum + weight_floor, times weight_scale."""
+        if scoring not in ("softmax_chosen", "sigmoid"):
+            raise ValueError("unknown scoring %r (known: softmax_chosen, sigmoid)" % (scoring,))
+        self.scoring, self.correction = scoring, bool(correction)
+        self.groups, self.keep_groups, self.group_top = int(groups), int(keep_groups), int(group_top)
+        self.weight_scale, self.weight_floor = float(weight_scale), float(weight_floor)
+        if scoring == "sigmoid":
+            E = int(num_experts)
+            if self.groups < 1 or E % self.groups or not 1 <= self.keep_groups <= self.groups \
+                    or int(top_k) > self.keep_groups * (E // self.groups) or not 1 <= self.group_top <= 4:
+                raise ValueError("%d experts in %d groups of which %d are kept cannot give %d choices"
+                                 % (E, self.groups, self.keep_groups, int(top_k)))
+        elif correction or self.groups != 1:
+            raise ValueError("a correction of the choice and groups of experts belong to the sigmoid scoring")
         self.hidden_size, self.num_experts, self.top_k = int(hidden_size), int(num_experts), int(top_k)
         self.expert_size = int(expert_size)
         self.shared_size = int(shared_size) if shared_size else 0
@@ -137,13 +156,15 @@ class RoutedGLU(Part):
             raise ValueError("routing takes 1 <= top_k <= experts <= %d, got top_k %d of %d experts"
                              % (ops.ROUTE_MAX_EXPERTS, self.top_k, self.num_experts))
         self.dtype, self.device = dtype, device
-        self.w_router = self.b_router = self.w_gate_up = self.w_down = None
+        self.w_router = self.b_router = self.w_gate_up = self.w_down = self.w_correction = None
 
     def weight_specs(self):
         H, F, S = self.hidden_size, self.expert_size, self.shared_size
         specs = {"router": WeightSpec((self.num_experts, H), std=0.2, keep_32bit=True)}
         if self.router_bias:
             specs["router.b"] = WeightSpec((self.num_experts,), std=0.2, keep_32bit=True)
+        if self.correction:
+            specs["correction"] = WeightSpec((self.num_experts,), std=0.2, keep_32bit=True)
         for e in range(self.num_experts):
             specs.update({"e%d.gate" % e: WeightSpec((F, H)), "e%d.up" % e: WeightSpec((F, H)),
                           "e%d.down" % e: WeightSpec((H, F))})
@@ -154,6 +175,7 @@ class RoutedGLU(Part):
     def bind_weights(self, t):
         self.w_router = t["router"].float().contiguous()
         self.b_router = t["router.b"].float().contiguous() if self.router_bias else None
+        self.w_correction = t["correction"].float().contiguous() if self.correction else None
         names = ["e%d" % e for e in range(self.num_experts)] + (["shared"] if self.shared_size else [])
         # every expert's gate rows, then its up rows: one expert's share of the stacked matrix is one piece
         self.w_gate_up = torch.cat([t[n + kind] for n in names for kind in (".gate", ".up")], dim=0).contiguous()
@@ -164,7 +186,11 @@ class RoutedGLU(Part):
 
     def route(self, x):
         """(ids int32 [T, top_k], weights float32 [T, top_k], the weights as rows over all experts [T, E])."""
-        return ops.route_topk(ops.router_scores(x, self.w_router, self.b_router), self.top_k)
+        z = ops.router_scores(x, self.w_router, self.b_router)
+        if self.scoring == "sigmoid":
+            return ops.route_sigmoid_groups(z, self.top_k, self.w_correction, self.groups, self.keep_groups, self.group_top,
+                                            True, self.weight_floor, self.weight_scale)
+        return ops.route_topk(z, self.top_k)
 
     def forward(self, x):
         ids, weights, dense = self.route(x)

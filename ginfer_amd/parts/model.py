@@ -74,6 +74,9 @@ class DecoderModel:
         # what happens to the stream where a group of layers is entered again (schedule entries say before which runs)
         self.reentry = (registry.lookup("reentry", spec.reentry.kind)(**spec.reentry.params, **kw)
                         if spec.reentry is not None else None)
+        # how the residual stream is kept where it is not one tensor [T, W] (several streams side by side), or None
+        self.stream = (registry.lookup("stream", spec.stream.kind)(**spec.stream.params, **kw)
+                       if spec.stream is not None else None)
         self.blocks = []
         for i, ls in enumerate(spec.layers):
             arrangement = registry.lookup("arrangement", ls.arrangement)
@@ -100,6 +103,8 @@ class DecoderModel:
 
     def _build(self, role, part_spec):
         params = dict(part_spec.params)
+        if "branches" in params:             # a part made of parts of its own family: built here, so that they share tables too
+            params["branches"] = [self._build(role, b) if hasattr(b, "kind") else b for b in params["branches"]]
         pos = params.get("position")
         if pos is not None and hasattr(pos, "kind"):
             key = pos.key()
@@ -116,6 +121,8 @@ class DecoderModel:
                (name_of("head"), self.head)]
         if self.reentry is not None:
             out.append((name_of("reentry"), self.reentry))
+        if self.stream is not None:
+            out.append((name_of("stream"), self.stream))
         for ls, block in zip(self.spec.layers, self.blocks):
             for role, part in block.parts():
                 out.append((_join(ls.prefix, ls.name_of(role)), part))     # a role spelt "" names its tensors in the layer itself
@@ -168,6 +175,8 @@ class DecoderModel:
     def forward(self, step):
         """Logits float32 [R, V] at `step.logit_rows`."""
         residual = self.embedding.forward(step.token_ids, step)
+        if self.stream is not None:
+            residual = self.stream.open(residual)
         delta = None
         prepared = None
         if self.reentry is not None:
@@ -184,6 +193,10 @@ class DecoderModel:
         for t in self.spec.tail_enter:
             delta = self._settle(residual, delta)
             residual = self.reentry.forward(residual, prepared, t)
+        if self.stream is not None:
+            if delta is not None:
+                raise ValueError("a block left its output pending behind the last run of a model with several streams")
+            return self.head.forward(self.final_norm.forward(self.stream.close(residual, step.logit_rows), None))
         n = self.final_norm.forward(residual, whole(delta, self.final_norm), rows=step.logit_rows)
         return self.head.forward(n)
 

@@ -3,7 +3,7 @@ reaches it, so no part knows which model it is in.  New kinds register themselve
 decorators below; the model builder looks kinds up here and nowhere else."""
 
 _REGISTRIES = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "embedding": {}, "head": {},
-               "arrangement": {}, "convolution": {}, "reentry": {}, "residual_gate": {}}
+               "arrangement": {}, "convolution": {}, "reentry": {}, "residual_gate": {}, "stream": {}, "connection": {}}
 
 
 def _register(role, kind):
@@ -47,6 +47,14 @@ def register_reentry(kind):
 
 def register_residual_gate(kind):
     return _register("residual_gate", kind)
+
+
+def register_stream(kind):
+    return _register("stream", kind)
+
+
+def register_connection(kind):
+    return _register("connection", kind)
 
 
 def register_arrangement(kind):

@@ -16,15 +16,20 @@ class RotaryNeoX(Part):
 
     style = "neox"
 
-    def __init__(self, theta, rotary_dim, max_positions, dtype=None, device=None, scaling=None, wide_frequencies=False):
+    def __init__(self, theta, rotary_dim, max_positions, dtype=None, device=None, scaling=None, wide_frequencies=False,
+                 linear_factor=None):
         """wide_frequencies: the frequencies are worked out in 64-bit and rounded to 32-bit once (else every step of
         their formula is 32-bit, as the reference has it).  scaling: None, or dict(factor, low, high, original): frequencies rescaled by their wavelength l = 2 pi / f
         (the scheme of the Llama 3.1 models): kept where l < original / high, divided by `factor` where l > original /
-        low, and between the two blended with s = (original / l - low) / (high - low): (1 - s) f / factor + s f."""
+        low, and between the two blended with s = (original / l - low) / (high - low): (1 - s) f / factor + s f.
+        linear_factor: every frequency is divided by it (positions stretched evenly), worked out in 64-bit."""
         if rotary_dim % 2 or rotary_dim <= 0:
             raise ValueError("rotary_dim must be positive and even, got %r" % (rotary_dim,))
         self.theta, self.rotary_dim, self.max_positions = float(theta), int(rotary_dim), int(max_positions)
-        self.wide_frequencies = bool(wide_frequencies) or scaling is not None
+        self.linear_factor = None if linear_factor is None else float(linear_factor)
+        if self.linear_factor is not None and not self.linear_factor > 0:
+            raise ValueError("linear_factor must be positive, got %r" % (linear_factor,))
+        self.wide_frequencies = bool(wide_frequencies) or scaling is not None or self.linear_factor is not None
         self.scaling = None if scaling is None else {k: float(scaling[k]) for k in ("factor", "low", "high", "original")}
         if self.scaling is not None and not (self.scaling["high"] > self.scaling["low"] > 0 and self.scaling["factor"] > 0
                                              and self.scaling["original"] > 0):
@@ -58,6 +63,8 @@ class RotaryNeoX(Part):
             elif wavelength >= sc["original"] / sc["high"]:
                 s = (sc["original"] / wavelength - sc["low"]) / (sc["high"] - sc["low"])
                 f = (1.0 - s) * f / sc["factor"] + s * f
+            if self.linear_factor is not None:
+                f = f / self.linear_factor
             out.append(f)
         return torch.tensor(out, dtype=torch.float64).to(torch.float32)
 
