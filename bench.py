@@ -112,6 +112,34 @@ PUGUZEN_SIZES = {"1.5b": (_puguzen_size(1536, 8960, 12, 2, 1024), TITOZEN_SIZES[
                  "7b": (_puguzen_size(3584, 18944, 28, 4, 2048), TITOZEN_SIZES["7b"][0])}
 
 
+# Layer sizes for the Nidasun design beside the Potupel design, the closest one the engine has (the same attention part with
+# a sink, a loop over the middle layers, the squared-relu and the routed feed-forward), at equal width, heads, runs and
+# vocabulary (--nidasun): four layers of which the two in the middle run twice (six runs): chunked attention with a learned
+# sink, lightning attention (heads 64 x 128), and twice a windowed attention beside a recurrent block as wide as the model, its
+# gates in one block per head; dense and routed feed-forwards in turn (8 experts in 4 groups of which 2 are kept, 2 chosen, each
+# a third as wide as the dense one); four residual streams.
+def _nidasun_size(width, ff, heads, kv_heads, span, vocab=32768):
+    rot = dict(base=500000.0, dims=64)
+    att = dict(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, rot=rot, mask=dict(size=span))
+    left = dict(att, rot=dict(rot, scaling=dict(factor=4.0)))
+    par = dict(left=left, right=dict(width=width, blocks=heads, conv=4), left_scale=1.0, right_scale=1.0)
+    third = -(-ff // 3 // 64) * 64
+    dense = dict(kind="dense", ff=ff)
+    moe = dict(kind="moe", router=dict(experts=8, top=2, scale=2.5, groups=dict(count=4, keep=2)), expert=dict(ff=third))
+    lit = dict(heads=heads, dim=64, vdim=128, decay=[1.0 - 2.0 ** (-5 - 4.0 * h / heads) for h in range(heads)])
+    return dict(architecture="Nidasun", vocab=vocab, width=width, norm=dict(eps=1e-5), streams=4, loop=dict(start=1, stop=3, times=2),
+                layers=[dict(type="attention", mixer=att, mlp=dense), dict(type="lightning", mixer=lit, mlp=moe),
+                        dict(type="parallel", mixer=par, mlp=dense), dict(type="parallel", mixer=par, mlp=moe)])
+
+
+NIDASUN_SIZES = {"1.5b": (_nidasun_size(1536, 8960, 12, 2, 1024), POTUPEL_SIZES["1.5b"][0]),
+                 "7b": (_nidasun_size(3584, 18944, 28, 4, 2048), POTUPEL_SIZES["7b"][0])}
+
+
+def compare_nidasun(args):
+    return compare_designs(args, "nidasun", "Nidasun", args.nidasun, NIDASUN_SIZES, beside=("potupel", "Potupel"))
+
+
 def compare_puguzen(args):
     return compare_designs(args, "puguzen", "Puguzen", args.puguzen, PUGUZEN_SIZES, beside=("titozen", "Titozen"))
 
@@ -237,6 +265,9 @@ def main():
     ap.add_argument("--puguzen", default=None, metavar="SIZES",
                     help="instead of the headline: the same comparison for the Puguzen design (comma-separated: %s), beside "
                          "the Titozen design at equal sizes" % ", ".join(sorted(PUGUZEN_SIZES)))
+    ap.add_argument("--nidasun", default=None, metavar="SIZES",
+                    help="instead of the headline: the same comparison for the Nidasun design (comma-separated: %s), beside "
+                         "the Potupel design at equal sizes" % ", ".join(sorted(NIDASUN_SIZES)))
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on ONE GPU; --gpus %d is not supported" % args.gpus)
@@ -253,6 +284,9 @@ def main():
         return
     if args.puguzen:
         print(json.dumps(compare_puguzen(args)))
+        return
+    if args.nidasun:
+        print(json.dumps(compare_nidasun(args)))
         return
 
     shape_name, shape = SHAPES[args.shape]

@@ -53,6 +53,9 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
   float rq[PER], rk[PER], ra[PER], rv;
   // q, k and v as the recurrence reads them: the projection's numbers, or their silu
   auto act = [&](float z) { return silu_inputs ? z / (1.0f + expf(-z)) : z; };
+  // without a rotation, the activation (and the scales behind it) waits until a tile is stored to LDS: the fetch runs a tile
+  // ahead, and nothing in it should use what its loads bring
+  const bool late = silu_inputs && rot_dims == 0;
   auto fetch = [&](int t0) {
     const int nt = min(TILE, n - t0);
 #pragma unroll
@@ -64,8 +67,8 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
         const int64_t row = first + t0 + tt;
         const float* qp = q + row * stride + h * dim;
         const float* kp = k + row * stride + h * dim;
-        qv = act(qp[i]);
-        kv = act(kp[i]);
+        qv = late ? qp[i] : act(qp[i]);
+        kv = late ? kp[i] : act(kp[i]);
         if (i < rot_dims) {
           const int f = i < half ? i : i - half, other = i < half ? i + half : i - half;
           const int64_t at = (int64_t)(start + t0 + tt) * half + f;
@@ -75,8 +78,10 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
           qv = i < half ? qv * c - qo * sn : qv * c + qo * sn;
           kv = i < half ? kv * c - ko * sn : kv * c + ko * sn;
         }
-        qv *= q_scale;
-        kv *= k_scale;
+        if (!late) {
+          qv *= q_scale;
+          kv *= k_scale;
+        }
         a = decay ? decay[row * hd + h * dim + i] : hdec;
       }
       rq[x] = qv;
@@ -84,7 +89,7 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
       ra[x] = a;
     }
     const int tt = threadIdx.x / DS_COLS, jj = threadIdx.x % DS_COLS;      // 16 * DS_COLS == DS_THREADS
-    rv = (tt < nt && v0 + jj < vdim) ? act(v[(int64_t)(first + t0 + tt) * stride + h * vdim + v0 + jj]) : 0.f;
+    rv = (tt < nt && v0 + jj < vdim) ? v[(int64_t)(first + t0 + tt) * stride + h * vdim + v0 + jj] : 0.f;
   };
   fetch(0);
   for (int t0 = 0; t0 < n; t0 += TILE) {
@@ -93,13 +98,13 @@ __global__ __launch_bounds__(DS_THREADS) void decay_scan_kernel(
 #pragma unroll
     for (int x = 0; x < PER; ++x) {
       const int idx = threadIdx.x + x * DS_THREADS;
-      qs[idx / DP][idx % DP] = rq[x];
-      ks[idx / DP][idx % DP] = rk[x];
+      qs[idx / DP][idx % DP] = late ? act(rq[x]) * q_scale : rq[x];
+      ks[idx / DP][idx % DP] = late ? act(rk[x]) * k_scale : rk[x];
       as[idx / DP][idx % DP] = ra[x];
     }
     {
       const int tt = threadIdx.x / DS_COLS, jj = threadIdx.x % DS_COLS;
-      if (tt < TILE) vs[tt][jj] = rv;
+      if (tt < TILE) vs[tt][jj] = act(rv);
     }
     __syncthreads();
     if (t0 + TILE < n) fetch(t0 + TILE);
@@ -209,6 +214,31 @@ __global__ __launch_bounds__(DS_THREADS) void head_norm_gate_kernel(T* __restric
   }
 }
 
+// the same for rows as wide as all heads together (a norm over the whole row): a workgroup a row
+template <typename T>
+__global__ __launch_bounds__(DS_THREADS) void wide_norm_gate_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                                                     const float* __restrict__ weight,
+                                                                     const float* __restrict__ gate, int64_t gate_stride,
+                                                                     int width, float eps, int sigmoid_gate) {
+  __shared__ float scratch[DS_THREADS / WAVE];
+  const int64_t t = blockIdx.x;
+  const float* p = x + t * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += DS_THREADS) ss = fmaf(p[i], p[i], ss);
+  ss = block_sum<DS_THREADS / WAVE>(ss, scratch);
+  const float rms = sqrtf(ss / (float)width + eps);
+  const float* g = gate ? gate + t * gate_stride : nullptr;
+  for (int i = threadIdx.x; i < width; i += DS_THREADS) {
+    float y = p[i] / rms;
+    if (weight) y *= weight[i];
+    if (g) {
+      const float z = g[i];
+      y *= (sigmoid_gate ? 1.0f : z) / (1.0f + expf(-z));
+    }
+    Num<T>::st(out + t * width + i, y);
+  }
+}
+
 extern "C" int ga_decay_scan(void* out, const void* q, const void* k, const void* v, int64_t stride, const void* decay,
                              const void* head_decay, const void* cos_t, const void* sin_t, int rot_dims, float q_scale,
                              float k_scale, void* state, const void* slots, const void* cu, const void* q_start, int entries,
@@ -252,6 +282,15 @@ extern "C" int ga_head_norm_gate(void* out, const void* x, const void* weight, c
                                  int weight_per_head, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (vdim <= 0 || heads <= 0) return -1;
+  if (heads == 1 && vdim >= 512 && tokens < (1ll << 31)) {          // a row of a wavefront's 64 lanes would be a long walk
+    if (out_bf16)
+      hipLaunchKernelGGL(wide_norm_gate_kernel<bf16_t>, dim3((unsigned)tokens), dim3(DS_THREADS), 0, stream, (bf16_t*)out,
+                         (const float*)x, (const float*)weight, (const float*)gate, gate_stride, vdim, eps, sigmoid_gate);
+    else
+      hipLaunchKernelGGL(wide_norm_gate_kernel<float>, dim3((unsigned)tokens), dim3(DS_THREADS), 0, stream, (float*)out,
+                         (const float*)x, (const float*)weight, (const float*)gate, gate_stride, vdim, eps, sigmoid_gate);
+    return GA_CHECK_LAUNCH();
+  }
   const int64_t rows = tokens * heads;
   const int per = DS_THREADS / WAVE;
   dim3 grid((unsigned)((rows + per - 1) / per)), block(DS_THREADS);

@@ -300,12 +300,13 @@ int ga_hc_sum_rows(void* out, const void* X, const void* rows, int n_rows, int w
 
 // ---- rglru.hip: the real-gated linear recurrent unit.  gates: a = exp(-rate * sigmoid(Ra u + ra) * softplus(lam)), b =
 // sqrt(1 - a^2) * sigmoid(Ri u + ri) * u, the matrices block-diagonal and handed over transposed [block][in][out]; all float
-// [tokens, channels].  scan: S_t = a_t S_(t-1) + b_t per channel over float state [slots, channels] (zeros where an entry's
-// q_start is 0), out = S * gelu_tanh(y), y float rows with a stride
+// [tokens, channels]; and g = gelu_tanh(y), y float rows with a stride.  scan: S_t = a_t S_(t-1) + b_t per channel over float
+// state [slots, channels] (zeros where an entry's q_start is 0), out = S * g
 int ga_rglru_gates(void* a_out, void* b_out, const void* u, const void* ra_t, const void* ra_b, const void* ri_t,
-                   const void* ri_b, const void* lam, int tokens, int channels, int blocks, float rate, hipStream_t stream);
-int ga_rglru_scan(void* out, const void* a, const void* b, const void* y, int64_t y_stride, void* state, const void* slots,
-                  const void* cu, const void* q_start, int entries, int channels, int out_bf16, hipStream_t stream);
+                   const void* ri_b, const void* lam, const void* y, int64_t y_stride, void* g_out, int tokens, int channels,
+                   int blocks, float rate, hipStream_t stream);
+int ga_rglru_scan(void* out, const void* a, const void* b, const void* g, void* state, const void* slots, const void* cu,
+                  const void* q_start, int entries, int tokens, int channels, int out_bf16, hipStream_t stream);
 
 // ---- random_fill.hip: out[i] = mean + std * normal(key, i) for n elements, float or bfloat16: the counter-based
 // generator of random_normal.h, which gives the host library (host/random_fill_host.cpp) the same bits

@@ -22,16 +22,56 @@ __global__ __launch_bounds__(HC_THREADS) void hc_open_kernel(float* __restrict__
   }
 }
 
+// V consecutive elements to a thread and access: 1, or 4 where the width allows it (16-byte accesses of the 32-bit rows, 8 or
+// 16 bytes of the compute dtype's)
+template <typename T, int V> struct Pack;
+template <> struct Pack<float, 1> {
+  static __device__ __forceinline__ void ld(const float* p, float (&v)[1]) { v[0] = *p; }
+  static __device__ __forceinline__ void st(float* p, const float (&v)[1]) { *p = v[0]; }
+};
+template <> struct Pack<bf16_t, 1> {
+  static __device__ __forceinline__ void ld(const bf16_t* p, float (&v)[1]) { v[0] = bf16_to_f32(*p); }
+  static __device__ __forceinline__ void st(bf16_t* p, const float (&v)[1]) { *p = f32_to_bf16(v[0]); }
+};
+template <> struct Pack<float, 4> {
+  static __device__ __forceinline__ void ld(const float* p, float (&v)[4]) {
+    const float4 f = *reinterpret_cast<const float4*>(p);
+    v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+  }
+  static __device__ __forceinline__ void st(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Pack<bf16_t, 4> {
+  static __device__ __forceinline__ void ld(const bf16_t* p, float (&v)[4]) {
+    const uint2 u = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(u.x << 16); v[1] = __uint_as_float(u.x & 0xffff0000u);
+    v[2] = __uint_as_float(u.y << 16); v[3] = __uint_as_float(u.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void st(bf16_t* p, const float (&v)[4]) {
+    uint2 u;
+    u.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+    u.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+  }
+};
+
 // u of a token in LDS (dynamic, `width` floats), then the norm's rows
-template <typename C>
+template <typename C, int V>
 __device__ __forceinline__ void hc_norm_rows(C* __restrict__ rows, const float* u, float ss, const float* __restrict__ gain,
                                              float eps, int width, int64_t t, float* scratch) {
   ss = block_sum<HC_THREADS / WAVE>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-  for (int c = threadIdx.x; c < width; c += HC_THREADS) Num<C>::st(rows + t * width + c, u[c] * inv * gain[c]);
+  for (int c = threadIdx.x * V; c < width; c += HC_THREADS * V) {
+    float g[V], r[V];
+    Pack<float, V>::ld(gain + c, g);
+#pragma unroll
+    for (int k = 0; k < V; ++k) r[k] = u[c + k] * inv * g[k];
+    Pack<C, V>::st(rows + t * width + c, r);
+  }
 }
 
-template <typename C>
+template <typename C, int V>
 __global__ __launch_bounds__(HC_THREADS) void hc_read_kernel(C* __restrict__ rows, const float* __restrict__ X,
                                                              const float* __restrict__ in_w, const float* __restrict__ gain,
                                                              float eps, int width, int streams) {
@@ -39,16 +79,27 @@ __global__ __launch_bounds__(HC_THREADS) void hc_read_kernel(C* __restrict__ row
   __shared__ float scratch[HC_THREADS / WAVE];
   const int64_t t = blockIdx.x;
   float ss = 0.f;
-  for (int c = threadIdx.x; c < width; c += HC_THREADS) {
-    float acc = 0.f;
-    for (int s = 0; s < streams; ++s) acc = fmaf(in_w[s], X[(t * streams + s) * width + c], acc);
-    u[c] = acc;
-    ss = fmaf(acc, acc, ss);
+  for (int c = threadIdx.x * V; c < width; c += HC_THREADS * V) {
+    float acc[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) acc[k] = 0.f;
+    for (int s = 0; s < streams; ++s) {
+      float x[V];
+      Pack<float, V>::ld(X + (t * streams + s) * width + c, x);
+      const float w = in_w[s];
+#pragma unroll
+      for (int k = 0; k < V; ++k) acc[k] = fmaf(w, x[k], acc[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      u[c + k] = acc[k];
+      ss = fmaf(acc[k], acc[k], ss);
+    }
   }
-  hc_norm_rows<C>(rows, u, ss, gain, eps, width, t, scratch);
+  hc_norm_rows<C, V>(rows, u, ss, gain, eps, width, t, scratch);
 }
 
-template <typename Y, typename C>
+template <typename Y, typename C, int V>
 __global__ __launch_bounds__(HC_THREADS) void hc_write_kernel(float* __restrict__ X, const float* __restrict__ mix,
                                                               const float* __restrict__ out_w, const Y* __restrict__ y,
                                                               int parts, int64_t part_stride, const float* __restrict__ next_in,
@@ -65,31 +116,51 @@ __global__ __launch_bounds__(HC_THREADS) void hc_write_kernel(float* __restrict_
   }
   __syncthreads();
   float ss = 0.f;
-  for (int c = threadIdx.x; c < width; c += HC_THREADS) {
-    float old[HC_MAX_STREAMS];
+  for (int c = threadIdx.x * V; c < width; c += HC_THREADS * V) {
+    float old[HC_MAX_STREAMS][V];
 #pragma unroll
-    for (int s = 0; s < HC_MAX_STREAMS; ++s) old[s] = s < streams ? X[(t * streams + s) * width + c] : 0.f;
-    float yv = Num<Y>::ld(y + t * width + c);
-    for (int p = 1; p < parts; ++p) yv += Num<Y>::ld(y + p * part_stride + t * width + c);
-    float acc = 0.f;
+    for (int s = 0; s < HC_MAX_STREAMS; ++s)
+      if (s < streams) Pack<float, V>::ld(X + (t * streams + s) * width + c, old[s]);
+    float yv[V];
+    Pack<Y, V>::ld(y + t * width + c, yv);
+    for (int p = 1; p < parts; ++p) {
+      float more[V];
+      Pack<Y, V>::ld(y + p * part_stride + t * width + c, more);
+#pragma unroll
+      for (int k = 0; k < V; ++k) yv[k] += more[k];
+    }
+    float acc[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) acc[k] = 0.f;
 #pragma unroll
     for (int j = 0; j < HC_MAX_STREAMS; ++j) {
       if (j < streams) {
-        float v = 0.f;
+        float v[V];
+#pragma unroll
+        for (int k = 0; k < V; ++k) v[k] = 0.f;
 #pragma unroll
         for (int s = 0; s < HC_MAX_STREAMS; ++s)
-          if (s < streams) v = fmaf(m[s * streams + j], old[s], v);
-        v = fmaf(o[j], yv, v);
-        X[(t * streams + j) * width + c] = v;
-        acc = fmaf(nin[j], v, acc);
+          if (s < streams) {
+#pragma unroll
+            for (int k = 0; k < V; ++k) v[k] = fmaf(m[s * streams + j], old[s][k], v[k]);
+          }
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          v[k] = fmaf(o[j], yv[k], v[k]);
+          acc[k] = fmaf(nin[j], v[k], acc[k]);
+        }
+        Pack<float, V>::st(X + (t * streams + j) * width + c, v);
       }
     }
     if (rows) {
-      u[c] = acc;
-      ss = fmaf(acc, acc, ss);
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        u[c + k] = acc[k];
+        ss = fmaf(acc[k], acc[k], ss);
+      }
     }
   }
-  if (rows) hc_norm_rows<C>(rows, u, ss, next_gain, next_eps, width, t, scratch);
+  if (rows) hc_norm_rows<C, V>(rows, u, ss, next_gain, next_eps, width, t, scratch);
 }
 
 __global__ __launch_bounds__(HC_THREADS) void hc_sum_rows_kernel(float* __restrict__ out, const float* __restrict__ X,
@@ -121,12 +192,12 @@ extern "C" int ga_hc_read(void* rows, const void* X, const void* in_w, const voi
   if (tokens <= 0) return 0;
   if (!hc_sizes_ok(width, streams)) return -1;
   const size_t lds = (size_t)width * sizeof(float);
-  if (rows_bf16)
-    hipLaunchKernelGGL(hc_read_kernel<bf16_t>, dim3(tokens), dim3(HC_THREADS), lds, stream, (bf16_t*)rows, (const float*)X,
-                       (const float*)in_w, (const float*)gain, eps, width, streams);
-  else
-    hipLaunchKernelGGL(hc_read_kernel<float>, dim3(tokens), dim3(HC_THREADS), lds, stream, (float*)rows, (const float*)X,
-                       (const float*)in_w, (const float*)gain, eps, width, streams);
+  const bool vec = width % 4 == 0 && (((uintptr_t)X | (uintptr_t)rows | (uintptr_t)gain) & 15) == 0;
+#define GO(C, V) hipLaunchKernelGGL((hc_read_kernel<C, V>), dim3(tokens), dim3(HC_THREADS), lds, stream, (C*)rows,          \
+                                    (const float*)X, (const float*)in_w, (const float*)gain, eps, width, streams)
+  if (rows_bf16) { if (vec) GO(bf16_t, 4); else GO(bf16_t, 1); }
+  else { if (vec) GO(float, 4); else GO(float, 1); }
+#undef GO
   return GA_CHECK_LAUNCH();
 }
 
@@ -137,11 +208,15 @@ extern "C" int ga_hc_write(void* X, const void* mix, const void* out_w, const vo
   if (!hc_sizes_ok(width, streams) || parts < 1 || (parts > 1 && y_bf16)) return -1;
   if ((rows != nullptr) != (next_in != nullptr) || (rows != nullptr) != (next_gain != nullptr)) return -2;
   const size_t lds = rows ? (size_t)width * sizeof(float) : 0;
-#define GO(Y, C) hipLaunchKernelGGL((hc_write_kernel<Y, C>), dim3(tokens), dim3(HC_THREADS), lds, stream, (float*)X,        \
-                                    (const float*)mix, (const float*)out_w, (const Y*)y, parts, part_stride,               \
-                                    (const float*)next_in, (const float*)next_gain, next_eps, (C*)rows, width, streams)
-  if (y_bf16) { if (rows_bf16) GO(bf16_t, bf16_t); else GO(bf16_t, float); }
-  else { if (rows_bf16) GO(float, bf16_t); else GO(float, float); }
+  const bool vec = width % 4 == 0 && (((uintptr_t)X | (uintptr_t)rows | (uintptr_t)next_gain | (uintptr_t)y) & 15) == 0 &&
+                   (part_stride * (y_bf16 ? 2 : 4)) % 16 == 0;
+#define GO(Y, C, V) hipLaunchKernelGGL((hc_write_kernel<Y, C, V>), dim3(tokens), dim3(HC_THREADS), lds, stream, (float*)X,  \
+                                       (const float*)mix, (const float*)out_w, (const Y*)y, parts, part_stride,            \
+                                       (const float*)next_in, (const float*)next_gain, next_eps, (C*)rows, width, streams)
+#define GV(Y, C) do { if (vec) GO(Y, C, 4); else GO(Y, C, 1); } while (0)
+  if (y_bf16) { if (rows_bf16) GV(bf16_t, bf16_t); else GV(bf16_t, float); }
+  else { if (rows_bf16) GV(float, bf16_t); else GV(float, float); }
+#undef GV
 #undef GO
   return GA_CHECK_LAUNCH();
 }

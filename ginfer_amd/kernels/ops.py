@@ -1645,11 +1645,12 @@ def hyper_sum(X, rows=None):
 RGLRU_MAX_BLOCK = 1920           # eight tokens' channels of a block lie in LDS
 
 
-def rglru_gates(u, ra_t, ra_bias, ri_t, ri_bias, lam, blocks, rate):
-    """u float32 [T, C] -> (a, b) float32 [T, C]: per block of C / blocks channels r = sigmoid(Ra u + ra), i = sigmoid(Ri u +
-    ri); a = exp(-rate * r * softplus(lam)); b = sqrt(1 - a^2) * i * u.  ra_t, ri_t: the blocks' square matrices transposed,
-    float32 [blocks, in, out]; the biases and lam float32 [C]."""
-    _dev(u, ra_t, ra_bias, ri_t, ri_bias, lam)
+def rglru_gates(u, ra_t, ra_bias, ri_t, ri_bias, lam, blocks, rate, y):
+    """u float32 [T, C] -> (a, b, g) float32 [T, C]: per block of C / blocks channels r = sigmoid(Ra u + ra), i = sigmoid(Ri u +
+    ri); a = exp(-rate * r * softplus(lam)); b = sqrt(1 - a^2) * i * u; g = gelu_tanh(y), y float32 [T, C] with unit inner
+    stride (columns of a projection, before their activation).  ra_t, ri_t: the blocks' square matrices transposed, float32
+    [blocks, in, out]; the biases and lam float32 [C]."""
+    _dev(u, ra_t, ra_bias, ri_t, ri_bias, lam, y)
     _need(u.dtype == torch.float32 and u.dim() == 2 and u.is_contiguous(), "u must be contiguous float32 [T, C]")
     T, C = u.shape
     _need(blocks >= 1 and C % blocks == 0 and C // blocks <= RGLRU_MAX_BLOCK, "%d channels in %d blocks (a block may hold up to %d)",
@@ -1659,28 +1660,28 @@ def rglru_gates(u, ra_t, ra_bias, ri_t, ri_bias, lam, blocks, rate):
         _f32(t, (blocks, bw, bw), name)
     for name, t in (("ra_bias", ra_bias), ("ri_bias", ri_bias), ("lam", lam)):
         _f32(t, (C,), name)
-    a = torch.empty((T, C), dtype=torch.float32, device=u.device)
-    b = torch.empty((T, C), dtype=torch.float32, device=u.device)
+    _need(y.dtype == torch.float32 and tuple(y.shape) == (T, C) and y.stride(1) == 1, "y must be float32 [%d, %d] with unit inner stride", T, C)
+    a, b, g = (torch.empty((T, C), dtype=torch.float32, device=u.device) for _ in range(3))
     _check(build.load("rglru").ga_rglru_gates(_ptr(a), _ptr(b), _ptr(u), _ptr(ra_t), _ptr(ra_bias), _ptr(ri_t), _ptr(ri_bias), _ptr(lam),
-                                              _i(T), _i(C), _i(blocks), _f(rate), _stream()), "rglru_gates")
-    return a, b
+                                              _ptr(y), _i64(y.stride(0)), _ptr(g), _i(T), _i(C), _i(blocks), _f(rate), _stream()),
+           "rglru_gates")
+    return a, b, g
 
 
-def rglru_scan(a, b, y, state, slots, step, dtype):
+def rglru_scan(a, b, g, state, slots, step, dtype):
     """S_t = a_t S_(t-1) + b_t per channel over the step's entries, from the state float32 [slots, C] (zeros where an entry's
-    q_start is 0), which moves on in place; returns S * gelu_tanh(y) in `dtype`, [T, C].  a, b float32 [T, C]; y float32 [T, C]
-    with unit inner stride (columns of a projection, before their activation)."""
-    _dev(a, b, y, state, slots)
+    q_start is 0), which moves on in place; returns S * g in `dtype`, [T, C].  a, b, g float32 [T, C]."""
+    _dev(a, b, g, state, slots)
     _need(a.dtype == torch.float32 and a.dim() == 2 and a.is_contiguous(), "a must be contiguous float32 [T, C]")
     T, C = a.shape
     _f32(b, (T, C), "b")
-    _need(y.dtype == torch.float32 and tuple(y.shape) == (T, C) and y.stride(1) == 1, "y must be float32 [%d, %d] with unit inner stride", T, C)
+    _f32(g, (T, C), "g")
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == C and state.is_contiguous(),
           "state must be contiguous float32 [slots, %d]", C)
     E = _step_entries(step, slots)
     _need(E <= 65535, "too many entries for one launch: %d", E)
     out = torch.empty((T, C), dtype=dtype, device=a.device)
-    _check(build.load("rglru").ga_rglru_scan(_ptr(out), _ptr(a), _ptr(b), _ptr(y), _i64(y.stride(0)), _ptr(state), _ptr(slots),
-                                             _ptr(step.cu_tokens), _ptr(step.q_start), _i(E), _i(C), _i(_is_bf16(dtype)), _stream()),
+    _check(build.load("rglru").ga_rglru_scan(_ptr(out), _ptr(a), _ptr(b), _ptr(g), _ptr(state), _ptr(slots), _ptr(step.cu_tokens),
+                                             _ptr(step.q_start), _i(E), _i(T), _i(C), _i(_is_bf16(dtype)), _stream()),
            "rglru_scan")
     return out

@@ -68,7 +68,14 @@ class HyperConnection(Part):
 
     @staticmethod
     def _gain(norm):
-        return norm.weight if norm.weight.dtype == torch.float32 else norm.weight.float()
+        """The norm's gain in 32-bit, converted once (a checkpoint may store it in the compute dtype)."""
+        if norm.weight.dtype == torch.float32:
+            return norm.weight
+        kept = getattr(norm, "_gain32", None)
+        if kept is None or kept[0] is not norm.weight:
+            kept = (norm.weight, norm.weight.float().contiguous())
+            norm._gain32 = kept
+        return kept[1]
 
     def read(self, X, norm):
         """The rows of `norm` (a gain over the root mean square) of what this sublayer reads."""

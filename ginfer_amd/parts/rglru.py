@@ -66,6 +66,6 @@ class RecurrentBlock(Part):
         proj = linear(x, self.w_in, self.b_in, out_dtype=torch.float32)
         u = ops.short_conv(proj[:, C:], self.w_conv, None if conv is None else conv.state, None if conv is None else conv.slots,
                            step, torch.float32, add_input=False, update=conv is not None and conv.owner, bias=self.b_conv)
-        a, b = ops.rglru_gates(u, self.ra_t, self.ra_b, self.ri_t, self.ri_b, self.lam, self.blocks, self.rate)
-        h = ops.rglru_scan(a, b, proj[:, :C], state.state, state.slots, step, self.dtype)
+        a, b, g = ops.rglru_gates(u, self.ra_t, self.ra_b, self.ri_t, self.ri_b, self.lam, self.blocks, self.rate, proj[:, :C])
+        h = ops.rglru_scan(a, b, g, state.state, state.slots, step, self.dtype)
         return linear(h, self.w_o, parts_ok=True)
