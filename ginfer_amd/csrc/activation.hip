@@ -211,31 +211,33 @@ extern "C" int ga_relu_square(void* out, const void* x, int64_t total, int is_bf
   return GA_CHECK_LAUNCH();
 }
 
-// Two results side by side, each with a factor: out[i] = sa * a[i] + sb * b[i], in 32-bit.  out may be a or b.
-template <typename T>
-__global__ __launch_bounds__(256) void scaled_sum_kernel(T* __restrict__ out, const T* __restrict__ a, const T* __restrict__ b,
-                                                         float sa, float sb, int64_t total) {
-  constexpr int V = 16 / sizeof(T);
-  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
-  if (i + V <= total) {
-    union { uint4 u; T e[V]; } x, y, o;
-    x.u = *reinterpret_cast<const uint4*>(a + i);
-    y.u = *reinterpret_cast<const uint4*>(b + i);
-#pragma unroll
-    for (int j = 0; j < V; ++j) Num<T>::st(&o.e[j], fmaf(sb, Num<T>::ld(&y.e[j]), sa * Num<T>::ld(&x.e[j])));
-    *reinterpret_cast<uint4*>(out + i) = o.u;
-  } else {
-    for (int64_t k = i; k < total; ++k) Num<T>::st(out + k, fmaf(sb, Num<T>::ld(b + k), sa * Num<T>::ld(a + k)));
+// Two results side by side, each with a factor: out[i] = sa * a[i] + sb * b[i], in 32-bit.  Each of a and b comes in the
+// output's dtype, or as the 32-bit partial sums [parts, total] of a product whose K was split (added in order first).
+// out may be a or b where that one is no partial sums.
+template <typename T, typename A, typename B>
+__global__ __launch_bounds__(256) void scaled_sum_kernel(T* __restrict__ out, const A* __restrict__ a, int a_parts,
+                                                         const B* __restrict__ b, int b_parts, float sa, float sb, int64_t total) {
+  const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  for (int64_t i = i0; i < i0 + 4 && i < total; ++i) {
+    float x = Num<A>::ld(a + i), y = Num<B>::ld(b + i);
+    for (int p = 1; p < a_parts; ++p) x += Num<A>::ld(a + p * total + i);
+    for (int p = 1; p < b_parts; ++p) y += Num<B>::ld(b + p * total + i);
+    Num<T>::st(out + i, fmaf(sb, y, sa * x));
   }
 }
 
-extern "C" int ga_scaled_sum(void* out, const void* a, const void* b, float sa, float sb, int64_t total, int is_bf16,
-                             hipStream_t stream) {
+extern "C" int ga_scaled_sum(void* out, const void* a, int a_parts, const void* b, int b_parts, float sa, float sb, int64_t total,
+                             int is_bf16, hipStream_t stream) {
   if (total <= 0) return 0;
-  if (((uintptr_t)out | (uintptr_t)a | (uintptr_t)b) % 16) return -1;
-  const int v = is_bf16 ? 8 : 4;
-  dim3 grid((unsigned)((total + 256 * v - 1) / (256 * v))), block(256);
-  if (is_bf16) hipLaunchKernelGGL(scaled_sum_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)a, (const bf16_t*)b, sa, sb, total);
-  else hipLaunchKernelGGL(scaled_sum_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)a, (const float*)b, sa, sb, total);
+  if (a_parts < 0 || b_parts < 0) return -1;
+  // parts == 0: the operand comes in the output's dtype; parts >= 1: 32-bit partial sums
+  dim3 grid((unsigned)((total + 1023) / 1024)), block(256);
+#define GO(T, A, B) hipLaunchKernelGGL((scaled_sum_kernel<T, A, B>), grid, block, 0, stream, (T*)out, (const A*)a, a_parts ? a_parts : 1, \
+                                       (const B*)b, b_parts ? b_parts : 1, sa, sb, total)
+#define GT(T) do { if (a_parts && b_parts) GO(T, float, float); else if (a_parts) GO(T, float, T); else if (b_parts) GO(T, T, float); \
+                   else GO(T, T, T); } while (0)
+  if (is_bf16) GT(bf16_t); else GT(float);
+#undef GT
+#undef GO
   return GA_CHECK_LAUNCH();
 }

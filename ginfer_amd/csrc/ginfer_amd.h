@@ -232,8 +232,10 @@ int ga_combine_pairs(void* out, const void* y, const void* shared, const void* w
 
 // ---- activation.hip: out[i] = max(x[i], 0)^2 over `total` elements (out may be x)
 int ga_relu_square(void* out, const void* x, int64_t total, int is_bf16, hipStream_t stream);
-// out[i] = sa * a[i] + sb * b[i] in 32-bit (two sublayers' results side by side); out may be a or b
-int ga_scaled_sum(void* out, const void* a, const void* b, float sa, float sb, int64_t total, int is_bf16, hipStream_t stream);
+// out[i] = sa * a[i] + sb * b[i] in 32-bit (two sublayers' results side by side).  a_parts / b_parts 0: the operand comes in
+// the output's dtype (out may be that operand); >= 1: float partial sums [parts, total], added in order first
+int ga_scaled_sum(void* out, const void* a, int a_parts, const void* b, int b_parts, float sa, float sb, int64_t total,
+                  int is_bf16, hipStream_t stream);
 
 // ---- decay_scan.hip: linear attention with a decay as a recurrence, S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per
 // head.  q, k, v: 32-bit rows with a common stride; a from `decay` float [tokens, heads dim] or from `head_decay` float

@@ -25,9 +25,9 @@ __device__ __forceinline__ float rg_gelu_tanh(float z) {
 
 // TOK tokens a thread; a workgroup holds `groups` such sets of tokens side by side where a part has fewer outputs than the
 // workgroup has threads (thread = (set of tokens, output)), so that all threads work and a part's matrices are read once for
-// groups * TOK tokens.  RG_BATCH elements of each matrix are asked for before the first is used.
-#define RG_BATCH 16
-template <int TOK>
+// groups * TOK tokens.  RG_BATCH elements of each matrix are asked for before the first is used: 16 in steps of many tokens,
+// 64 in steps of few (a decode step waits for nothing but these loads, one round after the other).
+template <int TOK, int RG_BATCH>
 __global__ __launch_bounds__(RG_THREADS) void rglru_gates_kernel(float* __restrict__ a_out, float* __restrict__ b_out,
                                                                  const float* __restrict__ u, const float* __restrict__ ra_t,
                                                                  const float* __restrict__ ra_b, const float* __restrict__ ri_t,
@@ -184,11 +184,12 @@ extern "C" int ga_rglru_gates(void* a_out, void* b_out, const void* u, const voi
   const size_t lds = (size_t)bw * groups * tok * sizeof(float);
   if (lds > 60 * 1024) return -2;
   dim3 grid((tokens + groups * tok - 1) / (groups * tok), blocks);
-#define GO(TOK) hipLaunchKernelGGL(rglru_gates_kernel<TOK>, grid, dim3(RG_THREADS), lds, stream, (float*)a_out, (float*)b_out,  \
+#define GO(TOK, B) hipLaunchKernelGGL((rglru_gates_kernel<TOK, B>), grid, dim3(RG_THREADS), lds, stream, (float*)a_out, (float*)b_out,  \
                                    (const float*)u, (const float*)ra_t, (const float*)ra_b, (const float*)ri_t,                \
                                    (const float*)ri_b, (const float*)lam, (const float*)y, y_stride, (float*)g_out, tokens,    \
                                    channels, blocks, groups, rate)
-  if (tok == 16) GO(16); else GO(8);
+  if (tokens <= 64) { if (tok == 16) GO(16, 64); else GO(8, 64); }
+  else { if (tok == 16) GO(16, 16); else GO(8, 16); }
 #undef GO
   return GA_CHECK_LAUNCH();
 }

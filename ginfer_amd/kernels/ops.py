@@ -1229,15 +1229,21 @@ def relu_square(x):
     return x
 
 
-def scaled_sum(a, b, sa, sb):
-    """sa * a + sb * b in 32-bit, written over a; a and b contiguous and alike (float32 or bfloat16)."""
+def scaled_sum(a, b, sa, sb, dtype):
+    """sa * a + sb * b in 32-bit, [T, W] in `dtype`.  Each of a and b is [T, W] in `dtype`, or float32 [parts, T, W]: the
+    partial sums of a product whose K was split, added in order first."""
     _dev(a, b)
-    _need(a.shape == b.shape and a.dtype == b.dtype and a.is_contiguous() and b.is_contiguous()
-          and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0, "a and b must be contiguous and alike at 16-byte addresses")
+    shape = tuple(a.shape[-2:])
+    parts = []
+    for name, t in (("a", a), ("b", b)):
+        _need(t.is_contiguous() and tuple(t.shape[-2:]) == shape and t.dim() in (2, 3), "%s must be contiguous [T, W] or [parts, T, W]", name)
+        _need(t.dtype == (torch.float32 if t.dim() == 3 else dtype), "%s: partial sums are float32, a whole result is %s", name, dtype)
+        parts.append(t.shape[0] if t.dim() == 3 else 0)
+    out = a if a.dim() == 2 else (b if b.dim() == 2 else torch.empty(shape, dtype=dtype, device=a.device))
     lib = build.load("activation")
-    _check(lib.ga_scaled_sum(_ptr(a), _ptr(a), _ptr(b), _f(sa), _f(sb), _i64(a.numel()), _i(_is_bf16(a.dtype)), _stream()),
-           "scaled_sum")
-    return a
+    _check(lib.ga_scaled_sum(_ptr(out), _ptr(a), _i(parts[0]), _ptr(b), _i(parts[1]), _f(sa), _f(sb), _i64(out.numel()),
+                             _i(_is_bf16(dtype)), _stream()), "scaled_sum")
+    return out
 
 
 def conv_rope_kv(proj, weight, state, slots, step, cos, sin, slot_mapping, k_pages, v_pages, num_heads, num_kv_heads, head_dim,

@@ -3,7 +3,6 @@ import torch
 
 from ..kernels import ops
 from .base import Part
-from .block import whole
 from .registry import register_mixer
 
 
@@ -54,8 +53,6 @@ class ParallelSum(Part):
         for b, (spec, n) in zip(self.branches, self._shares()):
             share = cache[at:at + n]
             at += n
-            r = b.forward(x, step, share if isinstance(spec, (list, tuple)) else share[0])
-            if r.dim() == 3:                 # partial sums of a K-split product
-                r = whole(r).to(self.dtype)
-            results.append(r)
-        return ops.scaled_sum(results[0], results[1], self.scales[0], self.scales[1])
+            # (a result may be the 32-bit partial sums of a product whose K was split: the sum's kernel adds them up)
+            results.append(b.forward(x, step, share if isinstance(spec, (list, tuple)) else share[0]))
+        return ops.scaled_sum(results[0], results[1], self.scales[0], self.scales[1], self.dtype)
