@@ -239,6 +239,58 @@ __global__ __launch_bounds__(DS_THREADS) void wide_norm_gate_kernel(T* __restric
   }
 }
 
+// the same for rows of a multiple of 4 up to DS_THREADS * 4 * PER elements: four consecutive elements a thread and access, all
+// of a row's operands asked for before the first is used; the sum of squares in the order of the kernel above (the same bits)
+template <typename T, int PER>
+__global__ __launch_bounds__(DS_THREADS) void wide_norm_gate_rows_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                                                          const float* __restrict__ weight,
+                                                                          const float* __restrict__ gate, int64_t gate_stride,
+                                                                          int width, float eps, int sigmoid_gate) {
+  __shared__ float scratch[DS_THREADS / WAVE];
+  const int64_t t = blockIdx.x;
+  float4 xv[PER], wv[PER], gv[PER];
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int i = 4 * (threadIdx.x + p * DS_THREADS);
+    if (i < width) {
+      xv[p] = *reinterpret_cast<const float4*>(x + t * width + i);
+      if (weight) wv[p] = *reinterpret_cast<const float4*>(weight + i);
+      if (gate) gv[p] = *reinterpret_cast<const float4*>(gate + t * gate_stride + i);
+    }
+  }
+  // a thread of the kernel above adds the squares of elements tid, tid + 256, ...; here it holds other elements, so the
+  // partial sums differ: rows of these widths always come here, never there
+  float ss = 0.f;
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int i = 4 * (threadIdx.x + p * DS_THREADS);
+    if (i < width) {
+      ss = fmaf(xv[p].x, xv[p].x, ss);
+      ss = fmaf(xv[p].y, xv[p].y, ss);
+      ss = fmaf(xv[p].z, xv[p].z, ss);
+      ss = fmaf(xv[p].w, xv[p].w, ss);
+    }
+  }
+  ss = block_sum<DS_THREADS / WAVE>(ss, scratch);
+  const float rms = sqrtf(ss / (float)width + eps);
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int i = 4 * (threadIdx.x + p * DS_THREADS);
+    if (i < width) {
+      float e[4] = {xv[p].x, xv[p].y, xv[p].z, xv[p].w};
+      const float w4[4] = {wv[p].x, wv[p].y, wv[p].z, wv[p].w};
+      const float g4[4] = {gv[p].x, gv[p].y, gv[p].z, gv[p].w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float y = e[k] / rms;
+        if (weight) y *= w4[k];
+        if (gate) y *= (sigmoid_gate ? 1.0f : g4[k]) / (1.0f + expf(-g4[k]));
+        Num<T>::st(out + t * width + i + k, y);
+      }
+    }
+  }
+}
+
 extern "C" int ga_decay_scan(void* out, const void* q, const void* k, const void* v, int64_t stride, const void* decay,
                              const void* head_decay, const void* cos_t, const void* sin_t, int rot_dims, float q_scale,
                              float k_scale, void* state, const void* slots, const void* cu, const void* q_start, int entries,
@@ -282,6 +334,17 @@ extern "C" int ga_head_norm_gate(void* out, const void* x, const void* weight, c
                                  int weight_per_head, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (vdim <= 0 || heads <= 0) return -1;
+  if (heads == 1 && vdim >= 512 && vdim % 4 == 0 && vdim <= DS_THREADS * 16 && tokens < (1ll << 31) && gate_stride % 4 == 0 &&
+      (((uintptr_t)x | (uintptr_t)weight | (uintptr_t)gate) & 15) == 0) {
+#define GW(T, PER) hipLaunchKernelGGL((wide_norm_gate_rows_kernel<T, PER>), dim3((unsigned)tokens), dim3(DS_THREADS), 0, stream,  \
+                                      (T*)out, (const float*)x, (const float*)weight, (const float*)gate, gate_stride, vdim, eps, \
+                                      sigmoid_gate)
+#define GT(T) do { if (vdim <= DS_THREADS * 4) GW(T, 1); else if (vdim <= DS_THREADS * 8) GW(T, 2); else GW(T, 4); } while (0)
+    if (out_bf16) GT(bf16_t); else GT(float);
+#undef GT
+#undef GW
+    return GA_CHECK_LAUNCH();
+  }
   if (heads == 1 && vdim >= 512 && tokens < (1ll << 31)) {          // a row of a wavefront's 64 lanes would be a long walk
     if (out_bf16)
       hipLaunchKernelGGL(wide_norm_gate_kernel<bf16_t>, dim3((unsigned)tokens), dim3(DS_THREADS), 0, stream, (bf16_t*)out,

@@ -11,7 +11,7 @@
 #include "ginfer_amd.h"
 
 #define HC_THREADS 256
-#define HC_MAX_STREAMS 8
+#define HC_MAX_STREAMS 16
 
 __global__ __launch_bounds__(HC_THREADS) void hc_open_kernel(float* __restrict__ X, const float* __restrict__ x, int width,
                                                              int streams) {
@@ -163,6 +163,91 @@ __global__ __launch_bounds__(HC_THREADS) void hc_write_kernel(float* __restrict_
   if (rows) hc_norm_rows<C, V>(rows, u, ss, next_gain, next_eps, width, t, scratch);
 }
 
+// The same for rows of up to HC_THREADS * 4 * PER elements and S streams known when compiled: all of a token's operands are
+// asked for before the first is used, the new u stays in registers, and the norm's gain is on its way during the sum through
+// LDS.  Every sum in the order of the kernel above: the same bits.  (A decode step's launch is a few trips to memory; this
+// one makes them two.)
+template <typename Y, typename C, int S, int PER>
+__global__ __launch_bounds__(HC_THREADS) void hc_write_rows_kernel(float* __restrict__ X, const float* __restrict__ mix,
+                                                                   const float* __restrict__ out_w, const Y* __restrict__ y,
+                                                                   int parts, int64_t part_stride,
+                                                                   const float* __restrict__ next_in,
+                                                                   const float* __restrict__ next_gain, float next_eps,
+                                                                   C* __restrict__ rows, int width) {
+  __shared__ float scratch[HC_THREADS / WAVE];
+  __shared__ float m[S * S], o[S], nin[S];
+  const int64_t t = blockIdx.x;
+  float old[PER][S][4], yv[PER][4], gain[PER][4];
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int c = 4 * (threadIdx.x + p * HC_THREADS);
+    if (c < width) {
+#pragma unroll
+      for (int s = 0; s < S; ++s) Pack<float, 4>::ld(X + (t * S + s) * width + c, old[p][s]);
+      Pack<Y, 4>::ld(y + t * width + c, yv[p]);
+      if (rows) Pack<float, 4>::ld(next_gain + c, gain[p]);
+    }
+  }
+  if (threadIdx.x < S * S) m[threadIdx.x] = mix[threadIdx.x];
+  if (threadIdx.x < S) {
+    o[threadIdx.x] = out_w[threadIdx.x];
+    nin[threadIdx.x] = next_in ? next_in[threadIdx.x] : 0.f;
+  }
+  for (int q = 1; q < parts; ++q) {
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+      const int c = 4 * (threadIdx.x + p * HC_THREADS);
+      if (c < width) {
+        float more[4];
+        Pack<Y, 4>::ld(y + q * part_stride + t * width + c, more);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) yv[p][k] += more[k];
+      }
+    }
+  }
+  __syncthreads();
+  float ss = 0.f, u[PER][4];
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int c = 4 * (threadIdx.x + p * HC_THREADS);
+    if (c < width) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) u[p][k] = 0.f;
+#pragma unroll
+      for (int j = 0; j < S; ++j) {
+        float v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = 0.f;
+#pragma unroll
+        for (int s2 = 0; s2 < S; ++s2)
+#pragma unroll
+          for (int k = 0; k < 4; ++k) v[k] = fmaf(m[s2 * S + j], old[p][s2][k], v[k]);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          v[k] = fmaf(o[j], yv[p][k], v[k]);
+          u[p][k] = fmaf(nin[j], v[k], u[p][k]);
+        }
+        Pack<float, 4>::st(X + (t * S + j) * width + c, v);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) ss = fmaf(u[p][k], u[p][k], ss);
+    }
+  }
+  if (!rows) return;
+  ss = block_sum<HC_THREADS / WAVE>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + next_eps);
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int c = 4 * (threadIdx.x + p * HC_THREADS);
+    if (c < width) {
+      float r[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) r[k] = u[p][k] * inv * gain[p][k];
+      Pack<C, 4>::st(rows + t * width + c, r);
+    }
+  }
+}
+
 __global__ __launch_bounds__(HC_THREADS) void hc_sum_rows_kernel(float* __restrict__ out, const float* __restrict__ X,
                                                                  const int32_t* __restrict__ rows, int width, int streams) {
   const int64_t r = blockIdx.x;
@@ -213,10 +298,20 @@ extern "C" int ga_hc_write(void* X, const void* mix, const void* out_w, const vo
 #define GO(Y, C, V) hipLaunchKernelGGL((hc_write_kernel<Y, C, V>), dim3(tokens), dim3(HC_THREADS), lds, stream, (float*)X,  \
                                        (const float*)mix, (const float*)out_w, (const Y*)y, parts, part_stride,            \
                                        (const float*)next_in, (const float*)next_gain, next_eps, (C*)rows, width, streams)
-#define GV(Y, C) do { if (vec) GO(Y, C, 4); else GO(Y, C, 1); } while (0)
+#define GR(Y, C, S, PER) hipLaunchKernelGGL((hc_write_rows_kernel<Y, C, S, PER>), dim3(tokens), dim3(HC_THREADS), 0, stream,   \
+                                            (float*)X, (const float*)mix, (const float*)out_w, (const Y*)y, parts, part_stride, \
+                                            (const float*)next_in, (const float*)next_gain, next_eps, (C*)rows, width)
+#define GP(Y, C, S) do { if (width <= HC_THREADS * 4) GR(Y, C, S, 1); else if (width <= HC_THREADS * 8) GR(Y, C, S, 2);         \
+                         else GR(Y, C, S, 4); } while (0)
+#define GV(Y, C) do { if (vec && width <= HC_THREADS * 16 && streams <= 4) {                                                   \
+                        if (streams == 1) GP(Y, C, 1); else if (streams == 2) GP(Y, C, 2);                                     \
+                        else if (streams == 3) GP(Y, C, 3); else GP(Y, C, 4);                                                  \
+                      } else if (vec) GO(Y, C, 4); else GO(Y, C, 1); } while (0)
   if (y_bf16) { if (rows_bf16) GV(bf16_t, bf16_t); else GV(bf16_t, float); }
   else { if (rows_bf16) GV(float, bf16_t); else GV(float, float); }
 #undef GV
+#undef GP
+#undef GR
 #undef GO
   return GA_CHECK_LAUNCH();
 }

@@ -43,12 +43,15 @@ __global__ __launch_bounds__(RG_THREADS) void rglru_gates_kernel(float* __restri
     us[i * per + tt] = tt < nt ? u[(int64_t)(t0 + tt) * channels + b * bw + i] : 0.f;
   }
   __syncthreads();
-  const int lanes = min(bw, RG_THREADS);               // outputs side by side in a workgroup
+  // a part's outputs may be dealt to several workgroups (gridDim.z: steps of few tokens, where a part's matrices are all
+  // that is read and more compute units should pull them)
+  const int os = (bw + gridDim.z - 1) / gridDim.z, o_begin = blockIdx.z * os, o_end = min(bw, o_begin + os);
+  const int lanes = min(os, RG_THREADS);               // outputs side by side in a workgroup
   const int tg = threadIdx.x / lanes;                  // this thread's set of tokens
   if (tg >= groups) return;
   const float* wa = ra_t + (int64_t)b * bw * bw;
   const float* wi = ri_t + (int64_t)b * bw * bw;
-  for (int o = threadIdx.x % lanes; o < bw; o += lanes) {
+  for (int o = o_begin + threadIdx.x % lanes; o < o_end; o += lanes) {
     float za[TOK], zi[TOK];
 #pragma unroll
     for (int tt = 0; tt < TOK; ++tt) za[tt] = zi[tt] = 0.f;
@@ -178,18 +181,27 @@ extern "C" int ga_rglru_gates(void* a_out, void* b_out, const void* u, const voi
   if (channels <= 0 || blocks <= 0 || channels % blocks || blocks > 65535) return -1;
   const int bw = channels / blocks;
   // sets of tokens side by side where a part is narrower than the workgroup (at most 8: the tile of u lies in LDS)
-  int groups = bw >= RG_THREADS ? 1 : RG_THREADS / bw;
+  // steps of few tokens: a part's outputs in slices of 32 to a workgroup (at most 16 slices)
+  int slices = 1;
+  if (tokens <= 64 && bw > 32) slices = (bw + 31) / 32 > 16 ? 16 : (bw + 31) / 32;
+  const int os = (bw + slices - 1) / slices;
+  int groups = os >= RG_THREADS ? 1 : RG_THREADS / os;
   if (groups > 8) groups = 8;
-  const int tok = (size_t)bw * groups * 16 * sizeof(float) <= 60 * 1024 ? 16 : 8;
+  int tok = 16;                                          // as many tokens a thread as leave the tile of u in 60 KB of LDS
+  while (tok > 1 && (size_t)bw * groups * tok * sizeof(float) > 60 * 1024) tok = tok > 4 ? tok / 2 : 1;
   const size_t lds = (size_t)bw * groups * tok * sizeof(float);
   if (lds > 60 * 1024) return -2;
-  dim3 grid((tokens + groups * tok - 1) / (groups * tok), blocks);
-#define GO(TOK, B) hipLaunchKernelGGL((rglru_gates_kernel<TOK, B>), grid, dim3(RG_THREADS), lds, stream, (float*)a_out, (float*)b_out,  \
+  while (groups > 1 && (groups - 1) * tok >= tokens) --groups;       // no more sets of tokens than the step has
+  const size_t lds2 = (size_t)bw * groups * tok * sizeof(float);
+  dim3 grid((tokens + groups * tok - 1) / (groups * tok), blocks, slices);
+#define GO(TOK, B) hipLaunchKernelGGL((rglru_gates_kernel<TOK, B>), grid, dim3(RG_THREADS), lds2, stream, (float*)a_out, (float*)b_out, \
                                    (const float*)u, (const float*)ra_t, (const float*)ra_b, (const float*)ri_t,                \
                                    (const float*)ri_b, (const float*)lam, (const float*)y, y_stride, (float*)g_out, tokens,    \
                                    channels, blocks, groups, rate)
-  if (tokens <= 64) { if (tok == 16) GO(16, 64); else GO(8, 64); }
-  else { if (tok == 16) GO(16, 16); else GO(8, 16); }
+  if (tok == 16) { if (tokens <= 64) GO(16, 64); else GO(16, 16); }
+  else if (tok == 8) { if (tokens <= 64) GO(8, 64); else GO(8, 16); }
+  else if (tok == 4) GO(4, 16);
+  else GO(1, 16);
 #undef GO
   return GA_CHECK_LAUNCH();
 }

@@ -1571,7 +1571,7 @@ def gated_residual_add(residual, z, y1, y2=None, next_gain=None, next_eps=0.0, d
 # ---------------------------------------------------------------------------------------------------------------------
 # hyper-connections: the residual stream as several streams side by side
 
-HYPER_MAX_STREAMS = 8
+HYPER_MAX_STREAMS = 16
 HYPER_MAX_WIDTH = 15360          # a token's row of 32-bit sums lies in LDS
 
 
@@ -1648,7 +1648,7 @@ def hyper_sum(X, rows=None):
 # ---------------------------------------------------------------------------------------------------------------------
 # the real-gated linear recurrent unit
 
-RGLRU_MAX_BLOCK = 1920           # eight tokens' channels of a block lie in LDS
+RGLRU_MAX_BLOCK = 15360          # one token's channels of a block lie in LDS (narrower blocks: up to 16 tokens a thread)
 
 
 def rglru_gates(u, ra_t, ra_bias, ri_t, ri_bias, lam, blocks, rate, y):

@@ -145,7 +145,7 @@ class _Step:
 def test_streams_opened_read_written_and_summed():
     from ginfer_amd.kernels import ops
     g = torch.Generator().manual_seed(0)
-    for streams, width in ((1, 7), (2, 96), (3, 328), (4, 1000), (8, 4100)):
+    for streams, width in ((1, 7), (2, 96), (3, 328), (4, 1000), (8, 4100), (16, 72)):
         x = torch.randn((5, width), generator=g) * 3
         X = ops.hyper_open(x.cuda(), streams)
         assert X.shape == (5, streams, width) and all(torch.equal(X[:, s].cpu(), x) for s in range(streams))
@@ -214,7 +214,7 @@ def test_recurrent_block_across_cuts_and_slots():
     g = torch.Generator().manual_seed(2)
     W, T = 56, 61
     cuts = [1, 1, 2, 5, 3, 16, 1, 31, 1]
-    for width, blocks, taps in ((40, 5, 3), (24, 1, 1), (64, 2, 4), (300, 3, 2)):
+    for width, blocks, taps in ((40, 5, 3), (24, 1, 1), (64, 2, 4), (300, 3, 2), (1200, 1, 2), (4000, 1, 3)):
         bw = width // blocks
         shapes = {"y": (width, W), "y.b": (width,), "x": (width, W), "x.b": (width,), "conv": (width, taps), "conv.b": (width,),
                   "ra": (blocks, bw, bw), "ra.b": (blocks, bw), "ri": (blocks, bw, bw), "ri.b": (blocks, bw), "lam": (width,),
@@ -238,6 +238,8 @@ def test_recurrent_block_across_cuts_and_slots():
                     # a second request's first tokens ride beside: its state lies in another slot
                     rows = torch.cat([x[at:at + n], other[:2 + i % 3]]).cuda().to(dt)
                     out = part.forward(rows, _Step([n, 2 + i % 3], [at, 0]), views)
+                    if out.dim() == 3:               # partial sums of a product whose K was split
+                        out = out.sum(0)
                     got.append(out[:n].float().cpu())
                     at += n
                 outs.append(torch.cat(got))
