@@ -70,10 +70,11 @@ class ConvAttention(Part):
         self.w_qkv = self.w_conv = self.w_o = self.sinks = self.b_qkv = self.b_o = self.qk_gain = None
 
     def cache_spec(self):
-        """[the convolution's state (or None), the pages of keys and values].  Chunks keep every page: the keys before a
-        token's chunk are never read again, but nothing gives them back before the request ends."""
+        """[the convolution's state (or None), the pages of keys and values].  With chunks the cache keeps what a window of
+        the chunk's length keeps: a token's own chunk starts inside that window, so every key it sees is held, and the
+        pages before it go back to the pool while the request runs."""
         state = StateSpec((self.taps - 1, self.width), torch.float32) if self.taps > 1 else None
-        return [state, KVCacheSpec(self.nkv, self.padded, self.window)]
+        return [state, KVCacheSpec(self.nkv, self.padded, self.window or self.chunk)]
 
     def weight_specs(self):
         n, H = self.names, self.hidden_size

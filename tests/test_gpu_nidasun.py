@@ -681,8 +681,8 @@ def test_greedy_generation_through_the_entry_point(folders, dtype):
 
 
 def test_pool_planned_from_the_device_memory(folders):
-    """No page counts given: the engine sizes the groups itself (every key of the chunked layer, the keys behind a window, state
-    slots) and generates what the plain statement generates."""
+    """No page counts given: the engine sizes the groups itself (the keys behind a window or inside a chunk, state slots) and
+    generates what the plain statement generates."""
     from ginfer_amd import Engine, EngineConfig, SamplingParams
     folder = folders["mix"]
     eng = Engine(EngineConfig(model_path=folder, dtype="float32", max_num_batched_tokens=64, max_num_seqs=4, max_seq_len=512,

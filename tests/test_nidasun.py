@@ -167,7 +167,7 @@ def test_tensor_names_shapes_and_caches():
     specs = model.cache_specs()
     assert len(specs) == 6                              # six runs: the looped layers keep a cache per pass
     none, kv = specs[0]
-    assert none is None and isinstance(kv, KVCacheSpec) and (kv.num_kv_heads, kv.head_dim, kv.window) == (2, 32, None)
+    assert none is None and isinstance(kv, KVCacheSpec) and (kv.num_kv_heads, kv.head_dim, kv.window) == (2, 32, 10)   # a chunk's length
     assert specs[1] == specs[3] == StateSpec((3, 8, 12), torch.float32)
     none, kv, state, conv = specs[2]
     assert none is None and (kv.num_kv_heads, kv.head_dim, kv.window) == (3, 16, 7)
@@ -187,7 +187,7 @@ def test_cache_manager_with_pages_and_state_of_every_run():
     cm.release("a")
     assert cm.can_append("b", 48) and cm.can_admit()
     cm.check()
-    # the two passes of the windowed layer hold places of their own in one group; the chunked layer keeps every page
+    # the two passes of the windowed layer hold places of their own in one group; the chunked layer's keys are another
     assert cm.group_of[(2, 1)][0] == cm.group_of[(4, 1)][0] and cm.group_of[(2, 1)] != cm.group_of[(4, 1)]
     assert cm.group_of[(0, 1)][0] != cm.group_of[(2, 1)][0]
 
