@@ -191,7 +191,7 @@ __global__ __launch_bounds__(DS_THREADS) void head_norm_gate_kernel(T* __restric
                                                                      const float* __restrict__ weight,
                                                                      const float* __restrict__ gate, int64_t gate_stride,
                                                                      int64_t rows, int heads, int vdim, float eps,
-                                                                     int sigmoid_gate, int weight_per_head) {
+                                                                     int sigmoid_gate) {
   const int64_t row = (int64_t)blockIdx.x * (DS_THREADS / WAVE) + threadIdx.x / WAVE;
   if (row >= rows) return;
   const int lane = threadIdx.x % WAVE;
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(DS_THREADS) void head_norm_gate_kernel(T* __restric
   const float* g = gate ? gate + t * gate_stride + (int64_t)h * vdim : nullptr;
   for (int i = lane; i < vdim; i += WAVE) {
     float y = p[i] / rms;
-    if (weight) y *= weight[weight_per_head ? (int64_t)h * vdim + i : i];
+    if (weight) y *= weight[i];
     if (g) {
       const float z = g[i];
       y *= (sigmoid_gate ? 1.0f : z) / (1.0f + expf(-z));
@@ -331,7 +331,7 @@ extern "C" int ga_gla_decay(void* decay, const void* low, int64_t low_stride, co
 
 extern "C" int ga_head_norm_gate(void* out, const void* x, const void* weight, const void* gate, int64_t gate_stride,
                                  int64_t tokens, int heads, int vdim, float eps, int out_bf16, int sigmoid_gate,
-                                 int weight_per_head, hipStream_t stream) {
+                                 hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (vdim <= 0 || heads <= 0) return -1;
   if (heads == 1 && vdim >= 512 && vdim % 4 == 0 && vdim <= DS_THREADS * 16 && tokens < (1ll << 31) && gate_stride % 4 == 0 &&
@@ -359,11 +359,9 @@ extern "C" int ga_head_norm_gate(void* out, const void* x, const void* weight, c
   dim3 grid((unsigned)((rows + per - 1) / per)), block(DS_THREADS);
   if (out_bf16)
     hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const float*)x,
-                       (const float*)weight, (const float*)gate, gate_stride, rows, heads, vdim, eps, sigmoid_gate,
-                       weight_per_head);
+                       (const float*)weight, (const float*)gate, gate_stride, rows, heads, vdim, eps, sigmoid_gate);
   else
     hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)x,
-                       (const float*)weight, (const float*)gate, gate_stride, rows, heads, vdim, eps, sigmoid_gate,
-                       weight_per_head);
+                       (const float*)weight, (const float*)gate, gate_stride, rows, heads, vdim, eps, sigmoid_gate);
   return GA_CHECK_LAUNCH();
 }

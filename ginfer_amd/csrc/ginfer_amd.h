@@ -250,9 +250,11 @@ int ga_decay_scan(void* out, const void* q, const void* k, const void* v, int64_
 // a2 transposed, float [rank, channels]
 int ga_gla_decay(void* decay, const void* low, int64_t low_stride, const void* a2t, const void* bias, int tokens,
                  int channels, int rank, float tau, hipStream_t stream);
-// out [tokens, heads, vdim] = x / rms(x over vdim) (* weight [vdim], or null) (* silu(gate), 32-bit rows with a stride, or null)
+// out [tokens, heads, vdim] = x / rms(x over vdim) (* weight [vdim], or null) (* silu(gate), or sigmoid(gate) where sigmoid_gate;
+// 32-bit rows with a stride, or null); heads == 1 with a wide vdim: a norm over all heads together
+// (decay_scan's silu_inputs: the recurrence reads silu(q), silu(k), silu(v))
 int ga_head_norm_gate(void* out, const void* x, const void* weight, const void* gate, int64_t gate_stride, int64_t tokens,
-                      int heads, int vdim, float eps, int out_bf16, int sigmoid_gate, int weight_per_head, hipStream_t stream);
+                      int heads, int vdim, float eps, int out_bf16, int sigmoid_gate, hipStream_t stream);
 
 // ---- pooled_attention.hip: attention over a window of tokens and the means of the blocks before it, sigmoid weights.
 // prepare: q and k of a 32-bit projection [q heads | k heads | v heads ...] turned by position (pairs 2i, 2i + 1), divided by

@@ -1400,7 +1400,7 @@ def head_norm_gate(x, weight, eps, dtype, proj=None, gate_start=0, sigmoid_gate=
     out = torch.empty((T, H * V), dtype=dtype, device=x.device)
     lib = build.load("decay_scan")
     _check(lib.ga_head_norm_gate(_ptr(out), _ptr(x), _ptr(weight), _ptr(gate), _i64(proj.stride(0) if proj is not None else 0),
-                                 _i64(T), _i(H), _i(V), _f(eps), _i(_is_bf16(dtype)), _i(1 if sigmoid_gate else 0), _i(0),
+                                 _i64(T), _i(H), _i(V), _f(eps), _i(_is_bf16(dtype)), _i(1 if sigmoid_gate else 0),
                                  _stream()), "head_norm_gate")
     return out
 
