@@ -192,6 +192,20 @@ def test_cache_manager_with_pages_and_state_of_every_run():
     assert cm.group_of[(0, 1)][0] != cm.group_of[(2, 1)][0]
 
 
+def test_the_kernels_mask_parameter_sees_what_the_plain_statement_sees():
+    """One signed number tells the attention kernels what a token sees; its host twin bounds the key splits."""
+    from ginfer_amd.kernels import ops
+    assert (ops.mask_parameter(), ops.mask_parameter(window=7), ops.mask_parameter(chunk=7)) == (0, 7, -7)
+    with pytest.raises(ops.KernelError):
+        ops.mask_parameter(window=3, chunk=3)
+    pos = torch.arange(40)
+    for kind, size, mask in (("chunk", 1, -1), ("chunk", 7, -7), ("chunk", 64, -64), ("window", 1, 1), ("window", 7, 7), ("all", 0, 0)):
+        seen = pn.visible(pos, kind, size)
+        for i in range(40):
+            first = ops.first_visible_key(i, mask)
+            assert seen[i].tolist() == [first <= j <= i for j in range(40)], (kind, size, i)
+
+
 def test_stretched_frequencies():
     part = RotaryNeoX(theta=100.0, rotary_dim=16, max_positions=32, linear_factor=2.0, device="cpu")
     cos, sin = part.tables()
